@@ -1,0 +1,127 @@
+/*
+ * psa_hip.h - C ABI of libpsa_hip.so: Pyramid Sparse Attention kernels for AMD MI355X (gfx950).
+ *
+ * The reference (ziplab/Pyramid-Sparse-Attention) has no FFI: its boundary is a set of Python
+ * callables that launch Triton kernels.  Each entry point below replaces one of those
+ * callables (cited as reference file:line); the Python package psa_hip binds them with ctypes
+ * and re-exposes the reference's names and signatures.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated or freed here;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*), no host synchronisation;
+ *   - return value 0 = ok, negative = error (see PSA_ERR_*); psa_last_error() gives a
+ *     thread-local human-readable message for the last failing call on this thread;
+ *   - activations are bf16, [B, H, L, D] with the D axis contiguous; batch/head/row strides are
+ *     given in elements (psa_tensor4), so transposed [B, L, H, D] views need no copy;
+ *   - D in {64, 128}; block_m in {64, 128}; block_n in {32, 64, 128};
+ *   - level maps hold one of {0, 1, 2, 4, 8} per (q-block, kv-block): 0 = skip, l = attend to the
+ *     kv-block's keys mean-pooled by l.  `map_elem_bytes` is 1 (int8) or 4 (int32, the reference's
+ *     dtype), layout [B, Hq, Mq, Nk] contiguous, Mq = ceil(L/block_m), Nk = ceil(L/block_n).
+ */
+#ifndef PSA_HIP_H
+#define PSA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PSA_OK 0
+#define PSA_ERR_ARG (-1)         /* null pointer, bad enum, bad size */
+#define PSA_ERR_UNSUPPORTED (-2) /* shape outside what the kernels are built for */
+#define PSA_ERR_LAUNCH (-3)      /* hip reported a launch error */
+
+#define PSA_MODE_TOPK 0
+#define PSA_MODE_THRESHOLDBOUND 1
+#define PSA_MAX_LEVEL_ITEMS 8
+
+typedef void* psa_stream_t; /* hipStream_t */
+
+/* [B, H, L, D] bf16 view; strides in elements; the D stride is 1. */
+typedef struct psa_tensor4 {
+  void* ptr;
+  int64_t stride_b;
+  int64_t stride_h;
+  int64_t stride_l;
+} psa_tensor4;
+
+int psa_version(void);
+const char* psa_last_error(void);
+
+/* Number of bf16 elements of one pooled buffer (levels 2, 4, 8 back to back):
+ * B*Hkv*Npad*D*7/8 with Npad = ceil(L/block_n)*block_n.  Level l starts at element
+ * psa_pool_level_offset(...) and is a contiguous [B, Hkv, Npad/l, D]. */
+int64_t psa_pool_elems(int B, int Hkv, int L, int D, int block_n);
+int64_t psa_pool_level_offset(int B, int Hkv, int L, int D, int block_n, int level);
+
+/* Pyramid pooling of K and V: one pass that reads K, V once and writes the 2x, 4x, 8x mean-pooled
+ * levels (each level rounded to bf16 before the next, tail replicate-padded to block_n).
+ * Replaces pad_to_multiple + pooling x3 per tensor:
+ *   reference src/psa_triton/kernels/psa_kernel.py:318-349,381-388
+ *   (same code at src/psa_triton/kernels/psa_kernel_legacy.py:806-834,868-875). */
+int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_pool,
+                int B, int Hkv, int L, int D, int block_n, psa_stream_t stream);
+
+/* Sampled block-importance estimate.  Row r of the sampled Q is source row
+ * min((r/keep_m)*block_m + off_q[b,h,r%keep_m], Lq-1) (off_q == NULL: offsets 0..keep_m-1, i.e. the
+ * input is already sampled when block_m == keep_m); rows past the last sampled row replicate it up to
+ * a multiple of 64, as the reference pads.  Same for K with off_k [B, Hkv, keep_n].
+ * scores [B, Hq, out_rows, out_cols] fp32 = rows normalised by the sum over ALL key groups
+ * (including the padding groups), cropped to out_rows x out_cols.
+ * Replaces _random_sample_tokens' gather + attn_with_pooling_optimized:
+ *   reference src/psa_triton/attention.py:116-137,178-223,
+ *   src/psa_triton/kernels/attn_pooling_kernel.py:12-116,119-282,285-451. */
+int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k,
+                         float* scores, int B, int Hq, int Hkv, int Lq, int Lk, int D,
+                         int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                         int out_rows, int out_cols, psa_stream_t stream);
+
+/* Scores -> level map.  One row = one (b, h, q-block).  Items are (level, upper bound) in the order
+ * the reference walks them: dict order for PSA_MODE_TOPK, ascending upper bound (stable) for
+ * PSA_MODE_THRESHOLDBOUND - the caller passes them already in that order.  align_div = block_n/tile_n.
+ * Writes map_out [rows, Nk] (map_elem_bytes 1 or 4; may be NULL) and/or list_out [rows, Nk+n_items]
+ * int32 (the reference's "new mask type" index list with -1 separators; may be NULL).
+ * Sort contract: descending, ties -> lower kv-block index; thresholdbound uses sequential fp64
+ * prefix sums rounded to fp32 and compares r <= fp32(hi + 1e-6).
+ * Replaces transfer_attn_to_mask: reference src/psa_triton/utils/transfer_attn_to_mask.py:6-507. */
+int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_t* list_out,
+                  int64_t rows, int Nk, int mode, int n_items, const int32_t* item_level,
+                  const double* item_hi, int align_div, int text_blocks, double min_full_attn_ratio,
+                  psa_stream_t stream);
+
+/* Index list ("new mask type", [rows, width] int32) -> dense level map [rows, Nk], read the way the
+ * reference's list-walking kernel reads it: segment level starts at 1, doubles at every -1, stops
+ * after 8.  reference src/psa_triton/kernels/psa_kernel.py:207-217. */
+int psa_map_from_list(const int32_t* list, void* map_out, int map_elem_bytes, int64_t rows,
+                      int width, int Nk, psa_stream_t stream);
+
+/* out[i] = min(map[i], cap[col]) with cap [B*Hkv... given per (b, h, kv-block)] broadcast over q-blocks:
+ * the "sim mask" clamp.  reference src/psa_triton/attention.py:296-299. */
+int psa_map_min_cap(void* map, int map_elem_bytes, const int32_t* cap, int64_t bh, int Mq, int Nk,
+                    psa_stream_t stream);
+
+/* mean(1/level) over the map, skipped blocks counting 0; causal != 0 counts lower-triangle pairs only.
+ * density_out: one float per (b, h) row of the [BH] vector, plus the overall mean at index BH.
+ * reference src/psa_triton/utils/transfer_attn_to_mask.py:510-544. */
+int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk, int causal,
+                float* density_out, psa_stream_t stream);
+
+/* Sparse attention forward from a level map.  out [B, Hq, L, D] bf16; lse (may be NULL)
+ * [B, Hq, L] fp32 = natural-log softmax denominator incl. the +ln(level) bias; map == NULL means
+ * dense attention (every pair at level 1; k_pool/v_pool may then be NULL).  K/V have Hkv heads,
+ * query head h uses kv head h / (Hq/Hkv).  causal != 0: kv-blocks above the diagonal are never
+ * visited and a pooled key t of level l is visible to query i iff (t+1)*l-1 <= i.
+ * Replaces the kernels behind sparse_attention_factory(...)(q, k, v, mask, sm_scale):
+ *   reference src/psa_triton/kernels/psa_kernel.py:24-316,351-457 (list walk, non-causal),
+ *   src/psa_triton/kernels/psa_kernel_legacy.py:34-799,837-938 (dense map, causal, L/M rows). */
+int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+            const void* map, int map_elem_bytes, psa_tensor4 out, float* lse,
+            int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
+            int causal, psa_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PSA_HIP_H */

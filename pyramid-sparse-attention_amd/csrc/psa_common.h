@@ -1,0 +1,73 @@
+// Shared device/host helpers for the PSA kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/psa_hip.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define PSA_WAVE 64
+
+// ---- host side: error reporting -------------------------------------------------------
+void psa_set_error(const char* fmt, ...);
+int psa_check_launch(const char* what);
+
+#define PSA_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) {                   \
+      psa_set_error(__VA_ARGS__);    \
+      return (code);                 \
+    }                                \
+  } while (0)
+
+static inline int psa_ilog2(int x) {
+  int r = 0;
+  while ((1 << r) < x) ++r;
+  return r;
+}
+static inline bool psa_is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+
+// ---- device side ----------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b16) { return __builtin_bit_cast(float, b16 << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bits (no NaN special-casing beyond keeping it a NaN)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  bf16_t h = (bf16_t)f;
+  return (uint32_t) __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  bf16x2 h = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, h);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ float shfl_xor32(float v) {
+  // exchange between the two 32-lane halves of a wave
+  return __shfl_xor(v, 32, 64);
+}
+
+// level value (0,1,2,4,8) of a map element of 1 or 4 bytes
+__device__ __forceinline__ int load_map(const void* map, int64_t idx, int elem_bytes) {
+  return elem_bytes == 1 ? (int)((const int8_t*)map)[idx] : ((const int32_t*)map)[idx];
+}
+__device__ __forceinline__ void store_map(void* map, int64_t idx, int elem_bytes, int v) {
+  if (elem_bytes == 1)
+    ((int8_t*)map)[idx] = (int8_t)v;
+  else
+    ((int32_t*)map)[idx] = v;
+}

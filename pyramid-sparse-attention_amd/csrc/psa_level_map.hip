@@ -1,0 +1,320 @@
+// Scores -> pyramid level map (and the index-list format), plus small map utilities.
+//
+// One workgroup per (b, h, q-block) row.  The row (<= a few thousand fp32 scores) lives in LDS:
+//   1. stable descending order by rank counting on a 64-bit key (inverted order-preserving score
+//      bits, then column index) - keys are unique so ties resolve to the lower column;
+//   2. thresholdbound only: sequential fp64 prefix sums rounded to fp32 (one lane walks the row,
+//      which keeps the additions in exactly the order a serial CPU scan uses), r = c / c[last] with
+//      an IEEE fp32 division, per-threshold counts of r <= thr;
+//   3. integer interval logic per item (alignment of each level's count to ceil(level/align_div));
+//   4. scatter of levels to their columns.
+// Latency-bound: about 1 KB read and 0.25-1 KB written per row.
+#include "psa_common.h"
+
+struct LevelMapParams {
+  const float* scores;
+  void* map_out;
+  int32_t* list_out;
+  int map_elem;
+  int Nk;
+  int mode;
+  int n_items;
+  int level[PSA_MAX_LEVEL_ITEMS];
+  int align[PSA_MAX_LEVEL_ITEMS];
+  float thr[PSA_MAX_LEVEL_ITEMS];     // thresholdbound: fp32(hi + 1e-6)
+  int fixed_s[PSA_MAX_LEVEL_ITEMS];   // topk: row-independent intervals
+  int fixed_e[PSA_MAX_LEVEL_ITEMS];
+  int min_index;                      // thresholdbound: floor for the level-1 interval
+  int text_blocks;
+};
+
+__device__ __forceinline__ uint32_t desc_key(float s) {
+  s += 0.0f;  // -0.0 -> +0.0 so that both zeros tie
+  uint32_t u = __builtin_bit_cast(uint32_t, s);
+  u ^= (u >> 31) ? 0xffffffffu : 0x80000000u;  // ascending order-preserving
+  return ~u;                                   // descending
+}
+
+__global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int N = p.Nk;
+  uint64_t* key = (uint64_t*)smem;            // [N]
+  float* sw = (float*)(key + N);              // [N] scores in sorted order
+  int* sidx = (int*)(sw + N);                 // [N] column of sorted position
+  float* c32 = (float*)(sidx + N);            // [N] prefix sums
+  __shared__ int s_cnt[PSA_MAX_LEVEL_ITEMS];
+  __shared__ int s_iv[PSA_MAX_LEVEL_ITEMS][2];
+
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t row = blockIdx.x;
+  const float* src = p.scores + row * N;
+
+  if (tid < PSA_MAX_LEVEL_ITEMS) s_cnt[tid] = 0;
+  for (int j = tid; j < N; j += nt) key[j] = ((uint64_t)desc_key(src[j]) << 32) | (uint32_t)j;
+  __syncthreads();
+  for (int j = tid; j < N; j += nt) {
+    const uint64_t kj = key[j];
+    int rank = 0;
+    for (int i = 0; i < N; ++i) rank += key[i] < kj ? 1 : 0;
+    sw[rank] = src[j];
+    sidx[rank] = j;
+  }
+  __syncthreads();
+
+  if (p.mode == PSA_MODE_THRESHOLDBOUND) {
+    if (tid == 0) {
+      double acc = 0.0;
+      for (int i = 0; i < N; ++i) {
+        acc += (double)sw[i];
+        c32[i] = (float)acc;
+      }
+    }
+    __syncthreads();
+    const float total = c32[N - 1];
+    int local[PSA_MAX_LEVEL_ITEMS];
+#pragma unroll
+    for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t) local[t] = 0;
+    for (int i = tid; i < N; i += nt) {
+      const float r = c32[i] / total;
+#pragma unroll
+      for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t)
+        if (t < p.n_items && r <= p.thr[t]) local[t]++;
+    }
+#pragma unroll
+    for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t)
+      if (t < p.n_items && local[t]) atomicAdd(&s_cnt[t], local[t]);
+    __syncthreads();
+    if (tid == 0) {
+      int last = 0;
+      for (int t = 0; t < p.n_items; ++t) {
+        const int cnt = s_cnt[t];
+        const int end0 = cnt > 0 ? cnt + 1 : last;
+        const int start = last;
+        const int al = p.align[t];
+        int end;
+        if (al > 1) {
+          int len = end0 - start;
+          len = len > 0 ? len : 0;
+          const int rem = len % al;
+          if (rem) len += al - rem;
+          end = start + len;
+          end = end < N ? end : N;
+          if (end == N) end = start + ((end - start) / al) * al;
+        } else {
+          end = end0 < 0 ? 0 : (end0 > N ? N : end0);
+          end = end > start ? end : start;
+          if (p.level[t] == 1) end = end > p.min_index ? end : p.min_index;
+        }
+        s_iv[t][0] = start;
+        s_iv[t][1] = end;
+        last = end;
+      }
+    }
+  } else {
+    if (tid < p.n_items) {
+      s_iv[tid][0] = p.fixed_s[tid];
+      s_iv[tid][1] = p.fixed_e[tid];
+    }
+  }
+  __syncthreads();
+
+  if (p.map_out) {
+    for (int i = tid; i < N; i += nt) {
+      int lv = 0;
+      for (int t = 0; t < p.n_items; ++t)
+        if (i >= s_iv[t][0] && i < s_iv[t][1]) lv = p.level[t];
+      const int col = sidx[i];
+      if (col >= N - p.text_blocks) lv = 1;
+      store_map(p.map_out, row * N + col, p.map_elem, lv);
+    }
+  }
+  if (p.list_out) {
+    const int W = N + p.n_items;
+    int32_t* dst = p.list_out + row * W;
+    for (int cidx = tid; cidx < W; cidx += nt) {
+      int v = 0;
+      for (int t = 0; t < p.n_items; ++t) {
+        const int pos = cidx - t;  // sorted position if this column belongs to segment t
+        if (pos >= s_iv[t][0] && pos < s_iv[t][1]) v = sidx[pos];
+        int sep = s_iv[t][1] + t;
+        sep = sep > W - 1 ? W - 1 : sep;
+        if (cidx == sep) v = -1;   // a separator written for item t survives later items' segments
+      }
+      dst[cidx] = v;
+    }
+  }
+}
+
+extern "C" int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_t* list_out, int64_t rows,
+                             int Nk, int mode, int n_items, const int32_t* item_level, const double* item_hi,
+                             int align_div, int text_blocks, double min_full_attn_ratio, psa_stream_t stream) {
+  PSA_REQUIRE(scores && (map_out || list_out), PSA_ERR_ARG, "psa_level_map: null pointer");
+  PSA_REQUIRE(item_level && item_hi, PSA_ERR_ARG, "psa_level_map: mask_ratios must be provided");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_level_map: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(mode == PSA_MODE_TOPK || mode == PSA_MODE_THRESHOLDBOUND, PSA_ERR_ARG,
+              "Unknown mode: %d. Must be 'topk' or 'thresholdbound'", mode);
+  PSA_REQUIRE(n_items >= 1 && n_items <= PSA_MAX_LEVEL_ITEMS, PSA_ERR_ARG, "psa_level_map: 1..%d items", PSA_MAX_LEVEL_ITEMS);
+  PSA_REQUIRE(rows > 0 && rows < (1ll << 31) && Nk > 0 && Nk <= 6144, PSA_ERR_UNSUPPORTED,
+              "psa_level_map: rows=%lld Nk=%d out of range (Nk <= 6144)", (long long)rows, Nk);
+  PSA_REQUIRE(align_div >= 1 && text_blocks >= 0, PSA_ERR_ARG, "psa_level_map: bad align_div/text_blocks");
+  LevelMapParams p;
+  p.scores = scores; p.map_out = map_out; p.list_out = list_out; p.map_elem = map_elem_bytes;
+  p.Nk = Nk; p.mode = mode; p.n_items = n_items;
+  p.text_blocks = text_blocks > Nk ? Nk : text_blocks;
+  int m = (int)((double)Nk * min_full_attn_ratio) + 1;
+  p.min_index = m < Nk ? m : Nk;
+  int last_end = 0;
+  for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t) {
+    p.level[t] = 0; p.align[t] = 1; p.thr[t] = 0.f; p.fixed_s[t] = 0; p.fixed_e[t] = 0;
+  }
+  for (int t = 0; t < n_items; ++t) {
+    const int lv = item_level[t];
+    PSA_REQUIRE(lv == 0 || lv == 1 || lv == 2 || lv == 4 || lv == 8, PSA_ERR_ARG, "psa_level_map: level %d not in {0,1,2,4,8}", lv);
+    p.level[t] = lv;
+    const int al = (lv + align_div - 1) / align_div;  // ceil(level / (block_n / tile_n)); 0 for the skip level
+    if (mode == PSA_MODE_THRESHOLDBOUND) {
+      p.align[t] = al;
+      p.thr[t] = (float)(item_hi[t] + 1e-6);
+    } else {
+      const int a = lv == 0 ? 1 : al;
+      const int start = last_end;
+      int end0 = (int)((double)Nk * item_hi[t]);
+      end0 = end0 < Nk ? end0 : Nk;
+      int end;
+      const int len = end0 - start;
+      if (a > 1 && len > 0) {
+        const int rem = len % a;
+        const int alen = rem ? len + (a - rem) : len;
+        end = start + alen < Nk ? start + alen : Nk;
+        if (end == Nk) end = start + ((end - start) / a) * a;
+      } else {
+        end = end0;
+      }
+      if (start < end) {
+        p.fixed_s[t] = start; p.fixed_e[t] = end; last_end = end;
+      } else {
+        p.fixed_s[t] = start; p.fixed_e[t] = start;
+      }
+    }
+  }
+  size_t shmem = (size_t)Nk * (8 + 4 + 4 + 4);
+  if (shmem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map: cannot reserve %zu bytes of LDS", shmem);
+  }
+  int nt = Nk <= 64 ? 64 : (Nk <= 128 ? 128 : 256);
+  hipLaunchKernelGGL(psa_level_map_kernel, dim3((unsigned)rows), dim3(nt), shmem, (hipStream_t)stream, p);
+  return psa_check_launch("psa_level_map");
+}
+
+// ---------------------------------------------------------------------------------------
+// index list -> dense map
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void psa_map_from_list_kernel(const int32_t* list, void* map, int map_elem, int width, int Nk) {
+  __shared__ int s_wave_sep[4];
+  const int64_t row = blockIdx.x;
+  const int32_t* src = list + row * width;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int j = tid; j < Nk; j += 256) store_map(map, row * Nk + j, map_elem, 0);
+  __syncthreads();
+  int seps_before = 0;  // separators in columns before the current chunk
+  for (int c0 = 0; c0 < width; c0 += 256) {
+    const int c = c0 + tid;
+    const int v = c < width ? src[c] : 0;
+    const bool is_sep = c < width && v == -1;
+    const uint64_t bal = __ballot(is_sep);
+    if (lane == 0) s_wave_sep[wave] = __popcll(bal);
+    __syncthreads();
+    int before = seps_before;
+    for (int w = 0; w < wave; ++w) before += s_wave_sep[w];
+    before += __popcll(bal & ((1ull << lane) - 1ull));
+    if (c < width && !is_sep && before <= 3 && v >= 0 && v < Nk) store_map(map, row * Nk + v, map_elem, 1 << before);
+    seps_before += s_wave_sep[0] + s_wave_sep[1] + s_wave_sep[2] + s_wave_sep[3];
+    __syncthreads();
+  }
+}
+
+extern "C" int psa_map_from_list(const int32_t* list, void* map_out, int map_elem_bytes, int64_t rows, int width, int Nk,
+                                 psa_stream_t stream) {
+  PSA_REQUIRE(list && map_out, PSA_ERR_ARG, "psa_map_from_list: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_map_from_list: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(rows > 0 && rows < (1ll << 31) && Nk > 0 && width >= Nk, PSA_ERR_ARG, "psa_map_from_list: bad sizes");
+  hipLaunchKernelGGL(psa_map_from_list_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, list, map_out,
+                     map_elem_bytes, width, Nk);
+  return psa_check_launch("psa_map_from_list");
+}
+
+// ---------------------------------------------------------------------------------------
+// map = min(map, cap[bh, col])
+// ---------------------------------------------------------------------------------------
+__global__ void psa_map_min_cap_kernel(void* map, int map_elem, const int32_t* cap, int Mq, int Nk) {
+  const int64_t bh = blockIdx.y;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)Mq * Nk) return;
+  const int col = (int)(i % Nk);
+  const int64_t idx = bh * Mq * Nk + i;
+  const int m = load_map(map, idx, map_elem);
+  const int c = cap[bh * Nk + col];
+  if (c < m) store_map(map, idx, map_elem, c);
+}
+
+extern "C" int psa_map_min_cap(void* map, int map_elem_bytes, const int32_t* cap, int64_t bh, int Mq, int Nk,
+                               psa_stream_t stream) {
+  PSA_REQUIRE(map && cap, PSA_ERR_ARG, "psa_map_min_cap: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_map_min_cap: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(bh > 0 && bh <= 65535 && Mq > 0 && Nk > 0, PSA_ERR_ARG, "psa_map_min_cap: bad sizes");
+  int64_t n = (int64_t)Mq * Nk;
+  hipLaunchKernelGGL(psa_map_min_cap_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0,
+                     (hipStream_t)stream, map, map_elem_bytes, cap, Mq, Nk);
+  return psa_check_launch("psa_map_min_cap");
+}
+
+// ---------------------------------------------------------------------------------------
+// density = mean(1/level)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void psa_density_kernel(const void* map, int map_elem, int Mq, int Nk, int causal, int BH,
+                                                          float* out) {
+  __shared__ float s_part[4];
+  const int64_t bh = blockIdx.x;
+  const int64_t n = (int64_t)Mq * Nk;
+  // counts per level are exact integers; 1/level sums are exact in fp32 up to 2^24/8 blocks
+  int c1 = 0, c2 = 0, c4 = 0, c8 = 0;
+  int64_t valid = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 256) {
+    const int r = (int)(i / Nk), c = (int)(i % Nk);
+    if (causal && c > r) continue;
+    ++valid;
+    const int lv = load_map(map, bh * n + i, map_elem);
+    c1 += lv == 1; c2 += lv == 2; c4 += lv == 4; c8 += lv == 8;
+  }
+  float v = (float)c1 + 0.5f * (float)c2 + 0.25f * (float)c4 + 0.125f * (float)c8;
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float tot = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    const double cnt = causal ? ((double)(Mq < Nk ? Mq : Nk) * ((Mq < Nk ? Mq : Nk) + 1) / 2.0 +
+                                 (Mq > Nk ? (double)(Mq - Nk) * Nk : 0.0))
+                              : (double)n;
+    const float d = (float)((double)tot / cnt);
+    out[bh] = d;
+  }
+}
+
+// overall mean in a fixed order (deterministic)
+__global__ void psa_density_mean_kernel(float* out, int BH) {
+  double acc = 0.0;
+  for (int i = 0; i < BH; ++i) acc += (double)out[i];
+  out[BH] = (float)(acc / (double)BH);
+}
+
+extern "C" int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk, int causal, float* density_out,
+                           psa_stream_t stream) {
+  PSA_REQUIRE(map && density_out, PSA_ERR_ARG, "psa_density: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_density: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(bh > 0 && bh < (1 << 30) && Mq > 0 && Nk > 0, PSA_ERR_ARG, "psa_density: bad sizes");
+  hipLaunchKernelGGL(psa_density_kernel, dim3((unsigned)bh), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes, Mq,
+                     Nk, causal, (int)bh, density_out);
+  hipLaunchKernelGGL(psa_density_mean_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, density_out, (int)bh);
+  return psa_check_launch("psa_density");
+}

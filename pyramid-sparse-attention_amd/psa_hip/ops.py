@@ -1,0 +1,253 @@
+"""Torch-facing wrappers of the C-ABI kernels.  PyTorch only supplies device memory and the
+current stream; every operator here runs a hand-written HIP kernel and there is no CPU path."""
+import ctypes
+from typing import Dict, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Tensor4, check, lib
+
+LEVELS = (1, 2, 4, 8)
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require_gpu(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("psa_hip operators run on the GPU only (got a %s tensor); there is no CPU path" % t.device)
+
+
+def _bf16_view(x: torch.Tensor) -> torch.Tensor:
+    """[B,H,L,D] tensor usable by the kernels: bf16, D contiguous, 16-byte aligned rows."""
+    if x.dim() != 4:
+        raise ValueError("expected a [B, H, L, D] tensor, got shape %s" % (tuple(x.shape),))
+    if x.dtype != torch.bfloat16:
+        x = x.to(torch.bfloat16)
+    ok = x.stride(3) == 1 and all(s % 8 == 0 for s in x.stride()[:3]) and x.data_ptr() % 16 == 0
+    return x if ok else x.contiguous()
+
+
+def _t4(x: torch.Tensor) -> Tensor4:
+    return Tensor4(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2))
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+# ----------------------------------------------------------------------------- pooling
+def pool_kv(k: torch.Tensor, v: torch.Tensor, block_n: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One pass over K and V -> flat pooled buffers holding levels 2, 4, 8 (see pool_levels)."""
+    _require_gpu(k, v)
+    k, v = _bf16_view(k), _bf16_view(v)
+    B, H, L, D = k.shape
+    if v.shape != k.shape:
+        raise ValueError("k and v must have the same shape")
+    n = lib.psa_pool_elems(B, H, L, D, block_n)
+    kp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+    vp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+    with torch.cuda.device(k.device):
+        check(lib.psa_pool_kv(_t4(k), _t4(v), _ptr(kp), _ptr(vp), B, H, L, D, block_n, _stream(k)), "psa_pool_kv")
+    return kp, vp
+
+
+def pool_levels(pool: torch.Tensor, B: int, H: int, L: int, D: int, block_n: int) -> Dict[int, torch.Tensor]:
+    """Views [B,H,Npad/l,D] of the levels inside a pooled buffer."""
+    npad = -(-L // block_n) * block_n
+    out = {}
+    for lv in (2, 4, 8):
+        off = lib.psa_pool_level_offset(B, H, L, D, block_n, lv)
+        n = B * H * (npad // lv) * D
+        out[lv] = pool[off:off + n].view(B, H, npad // lv, D)
+    return out
+
+
+# ----------------------------------------------------------------------------- estimator
+def estimate_sampled(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    off_q: Optional[torch.Tensor],
+    off_k: Optional[torch.Tensor],
+    block_m: int,
+    block_n: int,
+    keep_m: int,
+    keep_n: int,
+    sm_scale: Optional[float] = None,
+    out_rows: Optional[int] = None,
+    out_cols: Optional[int] = None,
+) -> torch.Tensor:
+    """fp32 block-importance scores [B,Hq,out_rows,out_cols]; off_* int32 [B,H,keep] in-block offsets
+    (None: rows are taken as 0..keep-1 of each block)."""
+    _require_gpu(q, k, off_q, off_k)
+    q, k = _bf16_view(q), _bf16_view(k)
+    B, Hq, Lq, D = q.shape
+    Hkv, Lk = k.shape[1], k.shape[2]
+    sm_scale = D ** -0.5 if sm_scale is None else sm_scale
+    Mq, Nk = -(-Lq // block_m), -(-Lk // block_n)
+    out_rows = Mq if out_rows is None else out_rows
+    out_cols = Nk if out_cols is None else out_cols
+    for o, H, keep in ((off_q, Hq, keep_m), (off_k, Hkv, keep_n)):
+        if o is not None and (o.dtype != torch.int32 or tuple(o.shape) != (B, H, keep) or not o.is_contiguous()):
+            raise ValueError("sample offsets must be contiguous int32 [B, H, keep]")
+    scores = torch.empty(B, Hq, out_rows, out_cols, dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        check(
+            lib.psa_estimate_sampled(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), B, Hq, Hkv, Lq, Lk, D,
+                                     block_m, block_n, keep_m, keep_n, float(sm_scale), out_rows, out_cols, _stream(q)),
+            "psa_estimate_sampled",
+        )
+    return scores
+
+
+# ----------------------------------------------------------------------------- level map
+def _items(mask_ratios, mode: str):
+    if mask_ratios is None:
+        raise ValueError("mask_ratios must be provided")
+    newtype = mode.endswith("_newtype")
+    base = mode[: -len("_newtype")] if newtype else mode
+    if base == "topk":
+        items = list(mask_ratios.items())
+        m = _lib.PSA_MODE_TOPK
+    elif base == "thresholdbound":
+        items = sorted(mask_ratios.items(), key=lambda x: x[1][1])
+        m = _lib.PSA_MODE_THRESHOLDBOUND
+    else:
+        raise ValueError(f"Unknown mode: {mode}. Must be 'topk' or 'thresholdbound'")
+    if len(items) > _lib.PSA_MAX_LEVEL_ITEMS:
+        raise ValueError("at most %d mask_ratios entries" % _lib.PSA_MAX_LEVEL_ITEMS)
+    return items, m, newtype
+
+
+def level_map(
+    scores: torch.Tensor,
+    mask_ratios,
+    text_length: int = 226,
+    mode: str = "topk",
+    min_full_attn_ratio: float = 0.06,
+    blocksize: int = 32,
+    compute_tile: int = 32,
+    map_dtype: torch.dtype = torch.int32,
+) -> torch.Tensor:
+    """Scores [B,H,Mq,Nk] -> level map (dense modes, `map_dtype` int8/int32) or int32 index list
+    (`*_newtype` modes)."""
+    items, m, newtype = _items(mask_ratios, mode)
+    _require_gpu(scores)
+    if scores.dim() != 4:
+        raise ValueError("scores must be [B, H, Mq, Nk]")
+    s = scores.to(torch.float32).contiguous()
+    B, H, Mq, Nk = s.shape
+    n = len(items)
+    lv = (ctypes.c_int32 * n)(*[int(i[0]) for i in items])
+    hi = (ctypes.c_double * n)(*[float(i[1][1]) for i in items])
+    rows = B * H * Mq
+    div = blocksize // compute_tile
+    if div < 1:
+        raise ValueError("compute_tile must not exceed blocksize")
+    with torch.cuda.device(s.device):
+        if newtype:
+            out = torch.empty(B, H, Mq, Nk + n, dtype=torch.int32, device=s.device)
+            rc = lib.psa_level_map(_ptr(s), None, 4, _ptr(out), rows, Nk, m, n, lv, hi, div, 0, float(min_full_attn_ratio), _stream(s))
+        else:
+            if map_dtype not in (torch.int8, torch.int32):
+                raise ValueError("map_dtype must be int8 or int32")
+            out = torch.empty(B, H, Mq, Nk, dtype=map_dtype, device=s.device)
+            tb = (text_length + blocksize - 1) // blocksize if text_length > 0 else 0
+            rc = lib.psa_level_map(_ptr(s), _ptr(out), out.element_size(), None, rows, Nk, m, n, lv, hi, div, tb,
+                                   float(min_full_attn_ratio), _stream(s))
+    check(rc, "psa_level_map")
+    return out
+
+
+def map_from_list(list_mask: torch.Tensor, Nk: int, map_dtype: torch.dtype = torch.int8) -> torch.Tensor:
+    """Index list [..., W] int32 -> dense level map [..., Nk]."""
+    _require_gpu(list_mask)
+    lm = list_mask.to(torch.int32).contiguous()
+    lead, W = lm.shape[:-1], lm.shape[-1]
+    rows = lm.numel() // W
+    out = torch.empty(*lead, Nk, dtype=map_dtype, device=lm.device)
+    with torch.cuda.device(lm.device):
+        check(lib.psa_map_from_list(_ptr(lm), _ptr(out), out.element_size(), rows, W, Nk, _stream(lm)), "psa_map_from_list")
+    return out
+
+
+def map_min_cap(level_map_: torch.Tensor, cap: torch.Tensor) -> torch.Tensor:
+    """In place: map[b,h,i,j] = min(map[b,h,i,j], cap[b,h,j])."""
+    _require_gpu(level_map_, cap)
+    B, H, Mq, Nk = level_map_.shape
+    if not level_map_.is_contiguous() or level_map_.dtype not in (torch.int8, torch.int32):
+        raise ValueError("level map must be a contiguous int8/int32 tensor")
+    cap = cap.to(torch.int32).contiguous()
+    if tuple(cap.shape) != (B, H, Nk):
+        raise ValueError("cap must be [B, H, Nk]")
+    with torch.cuda.device(level_map_.device):
+        check(lib.psa_map_min_cap(_ptr(level_map_), level_map_.element_size(), _ptr(cap), B * H, Mq, Nk, _stream(cap)), "psa_map_min_cap")
+    return level_map_
+
+
+def density(level_map_: torch.Tensor, causal: bool = False) -> torch.Tensor:
+    """Device-side mean(1/level): returns a float32 tensor [B*H + 1] (per (b,h), then the overall
+    mean) without synchronising the host."""
+    _require_gpu(level_map_)
+    m = level_map_.contiguous()
+    B, H, Mq, Nk = m.shape
+    out = torch.empty(B * H + 1, dtype=torch.float32, device=m.device)
+    with torch.cuda.device(m.device):
+        check(lib.psa_density(_ptr(m), m.element_size(), B * H, Mq, Nk, int(causal), _ptr(out), _stream(m)), "psa_density")
+    return out
+
+
+# ----------------------------------------------------------------------------- attention forward
+def sparse_attention_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    level_map_: Optional[torch.Tensor],
+    block_m: int,
+    block_n: int,
+    sm_scale: Optional[float] = None,
+    causal: bool = False,
+    return_lse: bool = False,
+    pools: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    out: Optional[torch.Tensor] = None,
+):
+    """Pyramid sparse attention forward.  level_map_ None = dense attention.  Returns out (dtype and
+    shape of q) or (out, lse fp32 [B,H,L], (k_pool, v_pool))."""
+    _require_gpu(q, k, v, level_map_)
+    in_dtype = q.dtype
+    qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
+    B, Hq, L, D = qb.shape
+    Hkv = kb.shape[1]
+    if kb.shape[2] != L or vb.shape != kb.shape or kb.shape[3] != D:
+        raise ValueError("q, k, v must share L and D; k and v must share their shape")
+    sm_scale = D ** -0.5 if sm_scale is None else float(sm_scale)
+    if not sm_scale > 0:
+        raise ValueError("sm_scale must be positive")
+    Mq, Nk = -(-L // block_m), -(-L // block_n)
+    kp = vp = None
+    if level_map_ is not None:
+        if level_map_.dtype not in (torch.int8, torch.int32):
+            level_map_ = level_map_.to(torch.int32)
+        level_map_ = level_map_.contiguous()
+        if tuple(level_map_.shape) != (B, Hq, Mq, Nk):
+            raise ValueError("level map must be [B, Hq, %d, %d], got %s" % (Mq, Nk, tuple(level_map_.shape)))
+        kp, vp = pools if pools is not None else pool_kv(kb, vb, block_n)
+    if out is None or out.dtype != torch.bfloat16:
+        o = torch.empty(B, Hq, L, D, dtype=torch.bfloat16, device=q.device)
+    else:
+        o = out
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
+    with torch.cuda.device(q.device):
+        check(
+            lib.psa_fwd(_t4(qb), _t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_),
+                        1 if level_map_ is None else level_map_.element_size(), _t4(o), _ptr(lse), B, Hq, Hkv, L, D,
+                        block_m, block_n, sm_scale, int(causal), _stream(q)),
+            "psa_fwd",
+        )
+    res = o if in_dtype == torch.bfloat16 else o.to(in_dtype)
+    if return_lse:
+        return res, lse, (kp, vp)
+    return res

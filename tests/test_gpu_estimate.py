@@ -1,0 +1,54 @@
+"""GPU parity of the sampled block-importance estimator against the oracle (fp32 scores from bf16
+inputs; both accumulate in fp32, so only the summation order differs)."""
+import numpy as np
+import pytest
+import torch
+
+import psa_oracle as O
+from gpu_util import dev, rnd
+
+pytestmark = pytest.mark.gpu
+RTOL = 2e-4  # fp32 scores; accumulation-order differences only
+
+
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,L,D,bm,bn",
+    [(1, 2, 2, 1024, 128, 128, 128), (2, 2, 1, 1000, 64, 128, 128), (1, 2, 2, 4096, 64, 64, 64), (1, 1, 1, 520, 128, 128, 32),
+     (1, 3, 3, 1111, 128, 128, 64), (1, 1, 1, 64, 64, 64, 64)],
+)
+def test_estimate_matches_oracle(B, Hq, Hkv, L, D, bm, bn):
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import sample_offsets
+
+    q, k = rnd(B, Hq, L, D, seed=1), rnd(B, Hkv, L, D, seed=2)
+    km, kn = bm // 4, bn // 4
+    oq, ok = sample_offsets(B, Hq, bm, km, 5), sample_offsets(B, Hkv, bn, kn, 6)
+    got = ops.estimate_sampled(q.to(dev()), k.to(dev()), oq.to(dev()), ok.to(dev()), bm, bn, km, kn)
+    ref = O.estimate_sampled(q, k, bm, bn, oq, ok)
+    assert got.shape == ref.shape and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), ref.numpy(), rtol=RTOL, atol=1e-9)
+
+
+def test_estimate_presampled_full_output_like_reference_api():
+    from psa_hip import ops
+
+    sq, sk = rnd(1, 2, 96, 128, seed=3), rnd(1, 2, 40, 128, seed=4)  # 96 -> 128 rows (4 groups of 32), 40 -> 64 keys (8 groups of 8)
+    ref = O.estimate_from_sampled(sq, sk, 128 ** -0.5, 32, 8)
+    got = ops.estimate_sampled(sq.to(dev()), sk.to(dev()), None, None, 32, 8, 32, 8, out_rows=4, out_cols=8)
+    np.testing.assert_allclose(got.cpu().numpy(), ref.numpy(), rtol=RTOL, atol=1e-9)
+    np.testing.assert_allclose(got.sum(-1).cpu().numpy(), 1.0, rtol=1e-5)
+
+
+def test_estimate_then_level_map_matches_oracle_map():
+    """The level map computed on the GPU from the GPU's own fp32 scores equals the oracle's map from
+    those same scores bit for bit (the map contract is defined on identical fp32 scores)."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    q, k, _ = make_qkv(1, 2, 2, (4, 16, 32), 128, seed=7)
+    oq, ok = sample_offsets(1, 2, 128, 32, 8), sample_offsets(1, 2, 128, 32, 9)
+    s = ops.estimate_sampled(q.to(dev()), k.to(dev()), oq.to(dev()), ok.to(dev()), 128, 128, 32, 32)
+    ratios = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
+    m = ops.level_map(s, ratios, 0, "thresholdbound", blocksize=128, compute_tile=32)
+    ref = O.level_map(s.cpu().numpy(), ratios, 0, "thresholdbound", blocksize=128, compute_tile=32)
+    assert np.array_equal(m.cpu().numpy(), ref)
