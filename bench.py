@@ -1,0 +1,223 @@
+"""Benchmark of the PSA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1] [--no-cpu]
+
+A step = one PSA attention layer over synthetic inputs already resident in HBM:
+pyramid pooling -> sampled block-importance estimate -> level map -> sparse attention forward.
+Prints ONE JSON line (metric of BASELINE.json) with a `roofline` object for the dominant kernel
+(the sparse forward, MFMA-bound) and a `cpu_baseline` object (the oracle on the host cores over a
+bounded sample of the same workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "pyramid-sparse-attention_amd")
+sys.path.insert(0, PKG)
+
+METRIC = "PSA attn ms/layer + effective TFLOPS (% bf16 MFMA peak) at Wan2.1-1.3B shape, 1 GPU"
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # BASELINE.json configs[1]: Wan2.1-1.3B 480p self-attention layer
+    "c2": dict(name="wan2.1-1.3b-480p B1 H12 N32760 D128 bf16 blk128 thresholdbound ~90% sparsity",
+               B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.90),
+    # BASELINE.json configs[0] (small; run in bf16 on the GPU)
+    "c1": dict(name="small B1 H2 N4096 D64 blk64 thresholdbound ~80% sparsity",
+               B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80),
+}
+WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
+
+
+def scaled_ratios(tau):
+    return {lv: (lo * tau if lv else 0.8 * tau, hi * tau if lv else 1.0) for lv, (lo, hi) in WAN13.items()}
+
+
+def time_gpu(fn, iters, warm=3):
+    import torch
+
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the path shards by (batch, head) with no exchange, "
+              "but nothing here launches more than one rank. Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not os.path.exists(os.path.join(PKG, "psa_hip", "libpsa_hip.so")):
+        import build_ext
+
+        build_ext.build(verbose=False)
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    w = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, D, bm, bn, tn = w["B"], w["H"], w["D"], w["bm"], w["bn"], w["tn"]
+    q, k, v = make_qkv(B, H, H, w["grid"], D, seed=args.seed, device=dev)
+    L = q.shape[2]
+    Mq, Nk = -(-L // bm), -(-L // bn)
+    km, kn = bm // 4, bn // 4
+    off_q = sample_offsets(B, H, bm, km, args.seed + 10, device=dev)
+    off_k = sample_offsets(B, H, bn, kn, args.seed + 11, device=dev)
+
+    # ---- calibrate tau so that sparsity ~= target (bisection on the level map, untimed) ----
+    scores = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
+    lo, hi = 0.05, 1.25
+    for _ in range(18):
+        tau = 0.5 * (lo + hi)
+        m = ops.level_map(scores, scaled_ratios(tau), 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
+        dens = float(ops.density(m)[-1])
+        if 1 - dens > w["sparsity"]:
+            lo = tau
+        else:
+            hi = tau
+    ratios = scaled_ratios(tau)
+
+    state = {}
+
+    def layer():
+        kp, vp = ops.pool_kv(k, v, bn)
+        s = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
+        mp = ops.level_map(s, ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
+        o = ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp))
+        state.update(kp=kp, vp=vp, s=s, mp=mp, o=o)
+        return o
+
+    # ---- the timed region: W warm-up steps, then exactly K steps --------------------------
+    for _ in range(args.warmup):
+        layer()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        layer()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_step = e0.elapsed_time(e1) / args.steps
+
+    mp, kp, vp = state["mp"], state["kp"], state["vp"]
+    density = float(ops.density(mp)[-1])
+    dense_flops = 4.0 * L * L * D * H * B
+    exec_flops = dense_flops * density
+
+    # ---- per-kernel timings (HIP events on the launch stream) ------------------------------
+    it = max(10, min(args.steps, 100))
+    t_pool, _ = time_gpu(lambda: ops.pool_kv(k, v, bn), it)
+    t_est, _ = time_gpu(lambda: ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn), it)
+    t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
+    out_buf = torch.empty_like(q)
+    t_fwd_med, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf), it)
+    t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
+    t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
+
+    pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
+    est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
+
+    roofline = {
+        "kernel": "psa_fwd_kernel",
+        "bound": "mfma",
+        "achieved": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12, 2),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+        "traffic": None,
+        "flops_per_launch": exec_flops,
+        "avg_launch_ms": round(t_fwd_avg, 4),
+    }
+
+    # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------
+    cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import psa_oracle as O
+
+        ncores = os.cpu_count() or 1
+        torch.set_num_threads(min(ncores, 32))
+        heads = [0, 1] if H >= 2 else [0]
+        qblocks = list(range(0, Mq, max(1, Mq // 32)))[:32]  # 32 evenly spaced q-blocks per sampled head
+        qc, kc, vc = (t[:, heads].float().cpu() for t in (q, k, v))
+        mc = mp[:, heads].cpu().numpy().astype("int32")
+        oqc, okc = off_q[:, heads].cpu(), off_k[:, heads].cpu()
+        t0c = time.perf_counter()
+        s_c = O.estimate_sampled(qc, kc, bm, bn, oqc, okc)
+        O.level_map(s_c.numpy(), ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn)
+        t_front = time.perf_counter() - t0c  # pooling is inside blockwalk
+        t1c = time.perf_counter()
+        O.psa_attention_blockwalk(qc, kc, vc, mc, bm, bn, qblocks=qblocks)
+        t_attn = (time.perf_counter() - t1c) * (Mq / len(qblocks))
+        cpu_s_per_layer = (t_front + t_attn) * (H / len(heads))
+        cpu = {
+            "value": round(dense_flops / cpu_s_per_layer / 1e12, 5),
+            "unit": "TFLOP/s (effective)",
+            "ms_per_layer": round(cpu_s_per_layer * 1e3, 1),
+            "cores": torch.get_num_threads(),
+            "host_cpus": ncores,
+            "kind": "port",
+            "sample": "heads %s of %d in fp32: full estimate + level map, attention on %d of %d q-blocks scaled to all; "
+                      "then scaled by H/%d" % (heads, H, len(qblocks), Mq, len(heads)),
+        }
+
+    eff_tflops = dense_flops / (ms_step * 1e-3) / 1e12
+    line = {
+        "metric": METRIC,
+        "value": round(eff_tflops, 2),
+        "unit": "effective TFLOP/s (dense-equivalent 4*N^2*D*H flops per layer / layer time)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded smooth 3-D field + noise, logit std ~3)",
+        "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
+                   "sparsity": round(1 - density, 4), "tau": round(tau, 4)},
+        "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
+                      "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4)},
+        "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),
+        "pct_bf16_peak_fwd_executed": round(100 * exec_flops / (t_fwd_med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
+        "pool_gbs": round(pool_bytes / (t_pool * 1e-3) / 1e9, 1),
+        "pool_pct_hbm": round(100 * pool_bytes / (t_pool * 1e-3) / 1e9 / PEAK_HBM_GBS, 2),
+        "estimate_tflops": round(est_flops / (t_est * 1e-3) / 1e12, 2),
+        "dense_fa": {"own_kernel_ms": round(t_dense, 3), "own_kernel_tflops": round(dense_flops / (t_dense * 1e-3) / 1e12, 1),
+                     "torch_sdpa_ms": round(t_sdpa, 3), "layer_speedup_vs_own_dense": round(t_dense / ms_step, 2),
+                     "layer_speedup_vs_sdpa": round(t_sdpa / ms_step, 2)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,217 @@
+"""Full-featured PSA module used by the diffusers attention processors:
+`attn.inner_attention(q, k, v, layer_idx)`.
+
+reference: src/psa_triton/pyramid_sparse_attention.py:28-83 (AttentionConfig), :139-249
+(estimate + mask + kernel), :252-413 (PyramidSparseAttention: warm-up steps, step counter,
+density logging, rearrangement hooks).
+"""
+import json
+import os
+import time
+from dataclasses import asdict, dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .attention import draw_sample_offsets
+from .kernels.calc_ksim_kernel import calc_k_similarity
+from .kernels.psa_kernel import sparse_attention_factory as psa_sparse_attention
+from .kernels.psa_kernel_legacy import sparse_attention_factory as psa_sparse_attention_legacy
+
+
+@dataclass
+class AttentionConfig:
+    """All tunables of the module (field names and defaults as in the reference)."""
+
+    # latent video grid and text tokens
+    width: int = 45
+    height: int = 30
+    depth: int = 13
+    text_length: int = 226
+    # attention
+    use_rearrange: bool = True
+    block_m: int = 32
+    block_n: int = 32
+    tile_n: int = 32
+    use_sim_mask: bool = True
+    mask_ratios: Dict[int, Tuple[float, float]] = None
+    mask_mode: str = "topk"
+    warmup_steps: int = 12
+    tile_size: Optional[Tuple[int, int, int]] = None
+    rearrange_method: str = None
+    attn_impl: str = "new_mask_type"
+    # logging
+    verbose: bool = False
+    enable_logging: bool = True
+    log_dir: str = "./psa_logs/"
+    # similarity thresholds of the sim mask
+    sim_2x_threshold: float = 0
+    sim_4x_threshold: float = 0
+    sim_8x_threshold: float = -1
+
+    def __post_init__(self):
+        if self.mask_ratios is None:
+            self.mask_ratios = {1: (0.0, 0.05), 2: (0.05, 0.15), 4: (0.15, 0.25), 8: (0.25, 0.5), 0: (0.5, 1.0)}
+        if self.attn_impl == "new_mask_type" and self.use_sim_mask:
+            raise ValueError(
+                "Incompatible configuration: 'new_mask_type' does not support 'use_sim_mask=True'.\n"
+                "Please choose one of the following options:\n"
+                "  1. Set 'use_sim_mask: false' to disable similarity mask\n"
+                "  2. Use 'attn_impl: old_mask_type' with block_size config (m=128, n=128, tile_n=32)"
+            )
+
+
+def efficient_attn_with_pooling(q, k, v, config, num_keep_m=32, num_keep_n=32, sample_offsets=None):
+    """Block importance [B,H,Mq,Nk] fp32 and the similarity cap [B,H,Nk] (or None).
+    reference: src/psa_triton/pyramid_sparse_attention.py:139-187."""
+    sim_cap = calc_k_similarity(k, config.block_n, config) if getattr(config, "use_sim_mask", True) else None
+    B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
+    if sample_offsets is None:
+        off_q = draw_sample_offsets(B, H, config.block_m, num_keep_m, q.device)
+        off_k = draw_sample_offsets(B, Hkv, config.block_n, num_keep_n, k.device)
+    else:
+        off_q, off_k = sample_offsets
+    pooling = ops.estimate_sampled(q, k, off_q, off_k, config.block_m, config.block_n, num_keep_m, num_keep_n, q.size(-1) ** -0.5)
+    return pooling, sim_cap
+
+
+def adaptive_block_sparse_attn(q, k, v, config, sparse_attention_fn, compute_stats=False, sample_offsets=None):
+    """estimate -> mask (-> min with the similarity cap) -> sparse attention.
+    Returns (out, sparsity, per_head_density, sim_cap); the statistics are device tensors
+    (no host synchronisation) unless compute_stats is False, in which case they are 0.0 / [].
+    reference: src/psa_triton/pyramid_sparse_attention.py:188-249."""
+    with torch.no_grad():
+        pooling, sim_cap = efficient_attn_with_pooling(q, k, v, config, config.block_m // 4, config.block_n // 4, sample_offsets)
+        if config.attn_impl == "old_mask_type":
+            mask = ops.level_map(pooling, config.mask_ratios, config.text_length, config.mask_mode, blocksize=config.block_n,
+                                 compute_tile=config.tile_n)
+        elif config.attn_impl == "new_mask_type":
+            mode = {"topk": "topk_newtype", "thresholdbound": "thresholdbound_newtype"}.get(config.mask_mode, "topk_newtype")
+            mask = ops.level_map(pooling, config.mask_ratios, config.text_length, mode, blocksize=config.block_n,
+                                 compute_tile=config.tile_n)
+        else:
+            raise ValueError(f"Unknown attn_impl: {config.attn_impl}")
+        if getattr(config, "use_sim_mask", True) and sim_cap is not None:
+            mask = ops.map_min_cap(mask, sim_cap)
+    out = sparse_attention_fn(q, k, v, mask, None)
+    if compute_stats:
+        dense = mask if config.attn_impl == "old_mask_type" else ops.map_from_list(mask, -(-k.shape[2] // config.block_n))
+        d = ops.density(dense)  # [B*H + 1] on the device
+        sparsity = 1 - d[-1]
+        per_head = d[:-1].view(q.shape[0], q.shape[1]).mean(0)
+    else:
+        sparsity, per_head = 0.0, []
+    return out, sparsity, per_head, sim_cap
+
+
+class _DensityLog:
+    """JSONL sparsity log: one line per layer call.  Values are kept as device tensors and only
+    brought to the host when the log is flushed, so logging does not synchronise every layer."""
+
+    def __init__(self, log_dir, config, model_type, layer_num, inference_num):
+        self.dir = os.path.join(log_dir, time.strftime("%Y%m%d_%H%M%S"))
+        os.makedirs(self.dir, exist_ok=True)
+        cfg = {k: (v if not isinstance(v, dict) else {str(a): list(b) for a, b in v.items()}) for k, v in asdict(config).items()}
+        with open(os.path.join(self.dir, "config.json"), "w") as f:
+            json.dump(dict(config=cfg, model_type=model_type, layer_num=layer_num, inference_num=inference_num), f, indent=1)
+        self.pending = []
+        self.closed = False
+
+    def log_sparsity(self, **kw):
+        self.pending.append(kw)
+        if len(self.pending) >= 256:
+            self.flush()
+
+    def flush(self):
+        if not self.pending:
+            return
+        with open(os.path.join(self.dir, "sparsity.jsonl"), "a") as f:
+            for rec in self.pending:
+                sp, ph = rec["sparsity"], rec["per_head_density"]
+                sp = float(sp) if torch.is_tensor(sp) else sp
+                ph = [float(x) for x in ph.cpu()] if torch.is_tensor(ph) else list(ph)
+                line = dict(layer_idx=rec["layer_idx"], sparsity=sp, density=1 - sp, per_head_density=ph,
+                            sequence_length=rec["sequence_length"], batch_size=rec["batch_size"], num_heads=rec["num_heads"],
+                            is_warmup=rec["is_warmup"])
+                f.write(json.dumps(line) + "\n")
+        self.pending = []
+
+    def close(self):
+        if not self.closed:
+            self.flush()
+            self.closed = True
+
+
+class PyramidSparseAttention(nn.Module):
+    """One instance is shared by every transformer block: forward(q, k, v, layer_idx)."""
+
+    def __init__(self, config: AttentionConfig = None, inference_num=50, layer_num=42, model_type="wan"):
+        super().__init__()
+        if config is None:
+            config = AttentionConfig()
+        self.config = config
+        self.model_type = model_type.lower()
+        self.rearranger = None
+        if config.use_rearrange:
+            if config.rearrange_method == "Gilbert":
+                from .utils.rearranger import GilbertRearranger
+
+                self.rearranger = GilbertRearranger(config.width, config.height, config.depth, config.text_length)
+            else:
+                raise NotImplementedError(
+                    f"rearrange_method={config.rearrange_method!r}: only 'Gilbert' (the method every shipped preset selects) is built"
+                )
+        self.sparsity_acc = 0.0
+        self.sparsity_counter = 0
+        self.use_rearrange = config.use_rearrange
+        self.inference_num = inference_num
+        self.layer_num = layer_num
+        self.sample_offsets = None
+        if config.attn_impl == "old_mask_type":
+            self.sparse_attention_fn = psa_sparse_attention_legacy(config.block_m, config.tile_n, config.block_n)
+        elif config.attn_impl == "new_mask_type":
+            self.sparse_attention_fn = psa_sparse_attention(config.block_m, config.tile_n, config.block_n)
+        else:
+            raise ValueError(f"Unknown attn_impl: {config.attn_impl}")
+        self.logger = None
+        if config.enable_logging:
+            self.logger = _DensityLog(config.log_dir, config, model_type, layer_num, inference_num)
+
+    def get_current_time(self):
+        """Denoising step index derived from the call counter (Wan runs cond + uncond per step)."""
+        if self.model_type == "cogvideo" or self.model_type == "wan2.1_1.3b_4steps":
+            return (self.sparsity_counter // self.layer_num) % self.inference_num
+        return (self.sparsity_counter // (2 * self.layer_num)) % self.inference_num
+
+    def forward(self, q, k, v, layer_idx):
+        if self.rearranger is not None:
+            q_r, k_r, v_r = self.rearranger.rearrange(q, k, v)
+        else:
+            q_r, k_r, v_r = q, k, v
+        is_warmup = self.get_current_time() < self.config.warmup_steps
+        compute_stats = self.config.verbose or self.logger is not None
+        if is_warmup:
+            out_r = ops.sparse_attention_fwd(q_r, k_r, v_r, None, 128, 128)  # dense attention, same kernel
+            sparsity = 0.0
+            per_head_density = [1.0] * q_r.shape[1] if compute_stats else []
+        else:
+            out_r, sparsity, per_head_density, _ = adaptive_block_sparse_attn(
+                q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets
+            )
+            if compute_stats:
+                self.sparsity_acc = self.sparsity_acc + sparsity
+        self.sparsity_counter += 1
+        if self.logger is not None:
+            self.logger.log_sparsity(layer_idx=layer_idx, sparsity=sparsity, per_head_density=per_head_density,
+                                     sequence_length=q.shape[2], batch_size=q.shape[0], num_heads=q.shape[1], is_warmup=is_warmup)
+        return self.rearranger.reversed_rearrange(out_r) if self.rearranger is not None else out_r
+
+    def close_logger(self):
+        if self.logger is not None:
+            self.logger.close()
+
+    def __del__(self):
+        if getattr(self, "logger", None) is not None:
+            self.logger.close()
