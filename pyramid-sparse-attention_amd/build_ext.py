@@ -39,7 +39,7 @@ def _run(cmd):
     return out
 
 
-def build(verbose=True):
+def build(verbose=True, extra_flags=(), out=OUT):
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
@@ -47,19 +47,19 @@ def build(verbose=True):
 
     def one(pair):
         s, o = pair
-        out = _run([hipcc, *FLAGS, "-c", s, "-o", o])
+        out = _run([hipcc, *FLAGS, *extra_flags, "-c", s, "-o", o])
         if verbose and out.strip():
             print(out)
         return o
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         list(ex.map(one, zip(srcs, objs)))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
     if verbose:
-        print("built", OUT)
-    return OUT
+        print("built", out)
+    return out
 
 
 if __name__ == "__main__":
-    build()
+    build(extra_flags=tuple(os.environ.get("PSA_EXTRA_HIPCC_FLAGS", "").split()))
     sys.exit(0)

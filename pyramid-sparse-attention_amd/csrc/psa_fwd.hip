@@ -3,8 +3,9 @@
 // One workgroup per (batch, head, q-block of BM = 32*NW rows); every wave owns 32 query rows.
 //
 //  * The workgroup first compacts its row of the level map into four per-level lists of kv-block
-//    ids in LDS (ballot + popcount, ascending block order - deterministic).
-//  * Work is then a sequence of TILES of 64 pooled keys of one level: a level-l kv-block holds
+//    ids in LDS (ballot + popcount, ascending block order - deterministic) and a list of tile
+//    descriptors.
+//  * Work is a sequence of TILES of 64 pooled keys of one level: a level-l kv-block holds
 //    block_n/l pooled keys, so one tile is half a 128-key block, one 64-key block, or 64/(block_n/l)
 //    small blocks of the same level packed side by side.  All tiles therefore cost the same MFMA
 //    work whatever their level; only the last tile of a level can be partly empty.
@@ -16,15 +17,20 @@
 //    holds 16 keys of ONE query column: the softmax row max / row sum are in-lane reductions plus a
 //    single exchange between the two half-waves, and P^T is already in B-operand layout (the
 //    key<->slot permutation it implies is applied to the V^T reads, which is free).
-//  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m).
-//  * Global loads of tile t+1 are issued before the math of tile t (register prefetch).
+//  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m); the running maximum is
+//    only raised when it grows by more than 2^8 would overflow nothing (lazy rescaling), so most
+//    tiles skip the accumulator rescale.
+//  * Software pipeline, one barrier per tile: while the softmax of tile t runs on the VALU the
+//    MFMA pipe computes S^T of tile t+1; K tiles t+2 and V tiles t+1 are written to the other LDS
+//    buffers and the global loads of K tile t+3 / V tile t+2 are in flight.
 //
 // Roofline: MFMA-bound; 4*BM*64*D flops per tile.
 #include "psa_common.h"
 
 namespace {
 
-constexpr int TK = 64;  // pooled keys per tile
+constexpr int TK = 64;              // pooled keys per tile
+constexpr float LAZY_THRESHOLD = 8.f;  // log2 units the running max may lag behind
 
 struct FwdParams {
   const bf16_t *q, *k, *v;
@@ -39,6 +45,7 @@ struct FwdParams {
   float scale_log2;
   int causal;
   int total_wg, wg_chunk;
+  int max_tiles;
 };
 
 template <int D>
@@ -48,30 +55,53 @@ struct Smem {
   static constexpr int K_BYTES = TK * KST;
   static constexpr int V_BYTES = D * VST;
   static constexpr int OST = D * 2 + 16;   // bytes per O staging row
-  static constexpr int tile_region(int bm) {  // K/V tiles and the O staging area share this region
-    return (K_BYTES + V_BYTES) > bm * OST ? (K_BYTES + V_BYTES) : bm * OST;
-  }
+  static constexpr int TILE_BYTES = 2 * K_BYTES + 2 * V_BYTES;  // double-buffered K and V^T
 };
 
-// source row (in the level's own row numbering) of tile slot r; returns -1 when the slot is empty
+// tile descriptor, word 0: level (2 bits) | masked (1) | nvalid 0..64 (7) | tile index inside the level (22)
+//                  word 1: offset of the level's block list (16) | number of blocks of the level (16)
+__device__ __forceinline__ u32x2 make_desc(int lv, bool masked, int nvalid, int lt, int ioff, int cnt) {
+  u32x2 d;
+  d[0] = (uint32_t)lv | ((uint32_t)masked << 2) | ((uint32_t)nvalid << 3) | ((uint32_t)lt << 10);
+  d[1] = (uint32_t)ioff | ((uint32_t)cnt << 16);
+  return d;
+}
+
+// Source row (in the level's own row numbering) of tile slot r, or -1 when the slot is empty.
+// The retained blocks of a level form one stream of cnt * 2^sbs_log2 pooled keys; tile lt covers
+// stream positions [64 lt, 64 lt + 64).
 __device__ __forceinline__ int slot_src(int lv, int lt, int r, int sbs_log2, int cnt, const uint16_t* ids, int L) {
-  int src;
-  if (sbs_log2 >= 6) {
-    const int tpb_log2 = sbs_log2 - 6;
-    const int bi = lt >> tpb_log2;
-    const int part = lt & ((1 << tpb_log2) - 1);
-    src = ((int)ids[bi] << sbs_log2) + (part << 6) + r;
-  } else {
-    const int bi = (lt << (6 - sbs_log2)) + (r >> sbs_log2);
-    if (bi >= cnt) return -1;
-    src = ((int)ids[bi] << sbs_log2) + (r & ((1 << sbs_log2) - 1));
-  }
-  if (lv == 0 && src >= L) return -1;
-  return src;
+  const int g = (lt << 6) + r;
+  const int bi = g >> sbs_log2;
+  if (bi >= cnt) return -1;
+  const int src = ((int)ids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
+  return (lv == 0 && src >= L) ? -1 : src;
 }
 
 template <int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
+#ifndef PSA_FWD_OCC
+#define PSA_FWD_OCC 2
+#endif
+__global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams p) {
+  // scalar copies of the arguments: lambdas below must not capture the argument struct itself
+  const auto P_B = p.B;
+  const auto P_Hkv = p.Hkv;
+  const auto P_L = p.L;
+  const auto P_bm = p.bm;
+  const auto P_bn_log2 = p.bn_log2;
+  const auto P_causal = p.causal;
+  const auto P_k = p.k;
+  const auto P_k_sb = p.k_sb;
+  const auto P_k_sh = p.k_sh;
+  const auto P_k_sl = p.k_sl;
+  const auto P_kp = p.kp;
+  const auto P_npad = p.npad;
+  const auto P_scale_log2 = p.scale_log2;
+  const auto P_v = p.v;
+  const auto P_v_sb = p.v_sb;
+  const auto P_v_sh = p.v_sh;
+  const auto P_v_sl = p.v_sl;
+  const auto P_vp = p.vp;
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
   constexpr int CH = D / 8;           // 16-byte chunks per row
@@ -80,12 +110,14 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
   constexpr int KK = D / 16;          // MFMA k-steps for QK^T
   constexpr int DB = D / 32;          // 32-row blocks of O^T
   using SM = Smem<D>;
+  static_assert(BM * SM::OST <= SM::TILE_BYTES, "O staging must fit the tile buffers");
 
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* Ks = smem;
-  unsigned char* Vt = smem + SM::K_BYTES;
-  uint16_t* ids = (uint16_t*)(smem + SM::tile_region(NW * 32));
-  __shared__ int s_cnt[4];
+  auto Kbuf = [&](int i) __attribute__((always_inline)) -> unsigned char* { return smem + (i & 1) * SM::K_BYTES; };
+  auto Vbuf = [&](int i) __attribute__((always_inline)) -> unsigned char* { return smem + 2 * SM::K_BYTES + (i & 1) * SM::V_BYTES; };
+  u32x2* tdesc = (u32x2*)(smem + SM::TILE_BYTES);
+  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
 
   // XCD-aware decode: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous range of (b, h, q-block) so that one XCD's L2 sees few heads at a time.
@@ -95,15 +127,15 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
   const int I = logical % p.Mq;
   const int bh = logical / p.Mq;
   const int h = bh % p.Hq, b = bh / p.Hq;
-  const int hk = h / (p.Hq / p.Hkv);
+  const int hk = h / (p.Hq / P_Hkv);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
 
   // ---- 1. compact the map row into per-level lists ------------------------------------
   int jmax = p.Nk;
-  if (p.causal) {
-    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << p.bn_log2) - 1) >> p.bn_log2);
+  if (P_causal) {
+    const int ce = (int)((((int64_t)(I + 1) * P_bm) + (1 << P_bn_log2) - 1) >> P_bn_log2);
     jmax = ce < jmax ? ce : jmax;
   }
   if (wave == 0) {
@@ -133,232 +165,258 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
         }
       }
     }
-    if (lane < 4) s_cnt[lane] = lane == 0 ? cnt[0] : lane == 1 ? cnt[1] : lane == 2 ? cnt[2] : cnt[3];
+    if (lane == 0) {
+      int io = 0, to = 0;
+#pragma unroll
+      for (int lv = 0; lv < 4; ++lv) {
+        const int c = lv == 0 ? cnt[0] : lv == 1 ? cnt[1] : lv == 2 ? cnt[2] : cnt[3];
+        const int sbs_log2 = P_bn_log2 - lv;
+        s_cnt[lv] = c;
+        s_ioff[lv] = io;
+        s_toff[lv] = to;
+        io += c;
+        to += sbs_log2 >= 6 ? (c << (sbs_log2 - 6)) : ((c << sbs_log2) + 63) >> 6;
+      }
+      s_toff[4] = to;
+    }
   }
 
   // ---- 2. Q fragments (B operand of S^T = K Q^T): lane holds Q[row l32][16*kk + 8*hh .. +8] ---
   const int q_row0 = I * BM + wave * 32;
+  const int q_idx = q_row0 + l32;
   bf16x8 qf[KK];
   {
-    int qr = q_row0 + l32;
-    qr = qr < p.L ? qr : p.L - 1;
+    const int qr = q_idx < P_L ? q_idx : P_L - 1;
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
   }
   __syncthreads();
 
-  int cnt[4], toff[5], ioff[4];
-  toff[0] = 0;
-  {
-    int io = 0;
-#pragma unroll
-    for (int lv = 0; lv < 4; ++lv) {
-      cnt[lv] = s_cnt[lv];
-      ioff[lv] = io;
-      io += cnt[lv];
-      const int sbs_log2 = p.bn_log2 - lv;
-      const int nt = sbs_log2 >= 6 ? (cnt[lv] << (sbs_log2 - 6)) : ((cnt[lv] << sbs_log2) + 63) >> 6;
-      toff[lv + 1] = toff[lv] + nt;
-    }
-  }
-  const int T = toff[4];
+  const int T = __builtin_amdgcn_readfirstlane(s_toff[4]);
 
-  // level bases
-  const bf16_t* kbase[4];
-  const bf16_t* vbase[4];
-  int64_t kstr[4], vstr[4];
-  kbase[0] = p.k + b * p.k_sb + hk * p.k_sh;
-  vbase[0] = p.v + b * p.v_sb + hk * p.v_sh;
-  kstr[0] = p.k_sl;
-  vstr[0] = p.v_sl;
-  {
-    const int64_t BH = (int64_t)p.B * p.Hkv;
-    const int64_t bhk = (int64_t)b * p.Hkv + hk;
-    int64_t off = 0;
-#pragma unroll
-    for (int lv = 1; lv < 4; ++lv) {
-      const int64_t n_l = p.npad >> lv;
-      kbase[lv] = p.kp + off + bhk * n_l * D;
-      vbase[lv] = p.vp + off + bhk * n_l * D;
-      kstr[lv] = D;
-      vstr[lv] = D;
-      off += BH * n_l * D;
+  // ---- 3. tile descriptors ------------------------------------------------------------------
+  for (int t = tid; t < T; t += NT) {
+    const int lv = (t >= s_toff[1]) + (t >= s_toff[2]) + (t >= s_toff[3]);
+    const int lt = t - s_toff[lv];
+    const int c_lv = s_cnt[lv];
+    const int io_lv = s_ioff[lv];
+    const int sbs_log2 = P_bn_log2 - lv;
+    // valid slots form a prefix of the tile: the level's stream ends, or (level 0) the sequence does
+    int nvalid = (c_lv << sbs_log2) - (lt << 6);
+    nvalid = nvalid < TK ? nvalid : TK;
+    const int last_blk = ids[io_lv + (((lt << 6) + nvalid - 1) >> sbs_log2)];
+    if (lv == 0) {
+      const int over = (((lt << 6) + nvalid - 1) & ((1 << sbs_log2) - 1)) + 1 - (P_L - (last_blk << sbs_log2));
+      if (over > 0) nvalid = nvalid - over > 0 ? nvalid - over : 0;
     }
+    const bool diag = P_causal && ((((int64_t)last_blk + 1) << P_bn_log2) - 1 > (int64_t)I * P_bm);
+    tdesc[t] = make_desc(lv, diag || nvalid < TK, nvalid, lt, io_lv, c_lv);
   }
 
-  auto tile_level = [&](int t) -> int { return t < toff[1] ? 0 : (t < toff[2] ? 1 : (t < toff[3] ? 2 : 3)); };
+  // level bases: level 0 is K/V itself; pooled level lv >= 1 starts npad - (npad >> (lv-1)) rows into the
+  // pooled buffer (all batches and heads of a level are contiguous)
+  const bf16_t* kb0 = P_k + b * P_k_sb + hk * P_k_sh;
+  const bf16_t* vb0 = P_v + b * P_v_sb + hk * P_v_sh;
+  const int64_t BHkv = (int64_t)P_B * P_Hkv, bhk = (int64_t)b * P_Hkv + hk;
 
-  u32x4 kreg[PER][4], vreg[PER][4];
-  auto load_tile = [&](int t) {
-    const int lv = tile_level(t);
-    const int lt = t - toff[lv];
-    const int sbs_log2 = p.bn_log2 - lv;
-    const bf16_t* kb = lv == 0 ? kbase[0] : (lv == 1 ? kbase[1] : (lv == 2 ? kbase[2] : kbase[3]));
-    const bf16_t* vb = lv == 0 ? vbase[0] : (lv == 1 ? vbase[1] : (lv == 2 ? vbase[2] : vbase[3]));
-    const int64_t ks = lv == 0 ? kstr[0] : D;
-    const int64_t vs = lv == 0 ? vstr[0] : D;
-    const int c = lv == 0 ? cnt[0] : (lv == 1 ? cnt[1] : (lv == 2 ? cnt[2] : cnt[3]));
-    const int io = lv == 0 ? ioff[0] : (lv == 1 ? ioff[1] : (lv == 2 ? ioff[2] : ioff[3]));
+  struct TileRef {
+    int lv, lt, cnt, sbs_log2;
+    const uint16_t* ids;
+    int64_t pool_off;
+  };
+  auto tile_ref = [&](int t) __attribute__((always_inline)) -> TileRef {
+    const u32x2 d = tdesc[t];
+    const uint32_t d0 = __builtin_amdgcn_readfirstlane(d[0]);
+    const uint32_t d1 = __builtin_amdgcn_readfirstlane(d[1]);
+    TileRef r;
+    r.lv = d0 & 3;
+    r.lt = d0 >> 10;
+    r.cnt = d1 >> 16;
+    r.ids = ids + (d1 & 0xffff);
+    r.sbs_log2 = P_bn_log2 - r.lv;
+    const int lm1 = r.lv > 0 ? r.lv - 1 : 0;
+    r.pool_off = (BHkv * (P_npad - (P_npad >> lm1)) + bhk * (P_npad >> r.lv)) * D;
+    return r;
+  };
+  // one (4 keys x 8 channels) unit per thread and PER
+  // Thread -> (key quad, 16-byte channel chunk) assignment.  K: neighbouring lanes walk along a row
+  // (whole 256-byte rows per 16 lanes).  V: neighbouring lanes walk along the key quads of one chunk,
+  // so that the transposed 8-byte LDS writes of 16 lanes fall into 16 different bank pairs.
+  auto unit_kq = [&](int u, bool vmap) __attribute__((always_inline)) { return vmap ? (u & 15) : (u / CH); };
+  auto unit_ch = [&](int u, bool vmap) __attribute__((always_inline)) { return vmap ? (u >> 4) : (u % CH); };
+  auto load_rows = [&](int t, const bf16_t* base0, int64_t str0, const bf16_t* pool, u32x4 (&reg)[PER][4], bool vmap) {
+    const TileRef r = tile_ref(t);
+    // uniform base pointer + 32-bit per-lane byte offset (a (b, h) slice is far below 4 GiB)
+    const char* base = (const char*)(r.lv == 0 ? base0 : pool + r.pool_off);
+    const uint32_t strb = r.lv == 0 ? (uint32_t)str0 * 2u : (uint32_t)(D * 2);
 #pragma unroll
     for (int u_ = 0; u_ < PER; ++u_) {
       const int u = tid + u_ * NT;
       if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u / CH) * 4, ch = u % CH;
-      const int src0 = slot_src(lv, lt, r0, sbs_log2, c, ids + io, p.L);  // 4 rows share a sub-block
+      const int r0 = unit_kq(u, vmap) * 4, ch = unit_ch(u, vmap);
+      // 4 rows share a sub-block.  Empty slots load row 0 of the level (finite data): their logits are
+      // masked to -inf, so they contribute exactly 0.
+      const int src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
+      const int lim = r.lv == 0 ? P_L : 0x7fffffff;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int src = src0 + i;
-        const bool ok = src0 >= 0 && (lv != 0 || src < p.L);
-        u32x4 z = {0u, 0u, 0u, 0u};
-        kreg[u_][i] = ok ? *(const u32x4*)(kb + (int64_t)src * ks + ch * 8) : z;
-        vreg[u_][i] = ok ? *(const u32x4*)(vb + (int64_t)src * vs + ch * 8) : z;
+        int src = src0 + i;
+        src = (src0 >= 0 && src < lim) ? src : 0;
+        reg[u_][i] = *(const u32x4*)(base + ((uint32_t)src * strb + (uint32_t)(ch * 16)));
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_k = [&](unsigned char* Ks, const u32x4 (&reg)[PER][4]) {
 #pragma unroll
     for (int u_ = 0; u_ < PER; ++u_) {
       const int u = tid + u_ * NT;
       if (UNITS % NT != 0 && u >= UNITS) break;
       const int r0 = (u / CH) * 4, ch = u % CH;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) *(u32x4*)(Ks + (r0 + i) * SM::KST + ch * 16) = kreg[u_][i];
+      for (int i = 0; i < 4; ++i) *(u32x4*)(Ks + (r0 + i) * SM::KST + ch * 16) = reg[u_][i];
+    }
+  };
+  auto store_vt = [&](unsigned char* Vt, const u32x4 (&reg)[PER][4]) {
+#pragma unroll
+    for (int u_ = 0; u_ < PER; ++u_) {
+      const int u = tid + u_ * NT;
+      if (UNITS % NT != 0 && u >= UNITS) break;
+      const int r0 = unit_kq(u, true) * 4, ch = unit_ch(u, true);
       // transpose 4 keys x 8 channels -> 8 channels x 4 keys
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         u32x2 e0, e1;
-        e0[0] = __builtin_amdgcn_perm(vreg[u_][1][j], vreg[u_][0][j], 0x05040100u);
-        e0[1] = __builtin_amdgcn_perm(vreg[u_][3][j], vreg[u_][2][j], 0x05040100u);
-        e1[0] = __builtin_amdgcn_perm(vreg[u_][1][j], vreg[u_][0][j], 0x07060302u);
-        e1[1] = __builtin_amdgcn_perm(vreg[u_][3][j], vreg[u_][2][j], 0x07060302u);
+        e0[0] = __builtin_amdgcn_perm(reg[u_][1][j], reg[u_][0][j], 0x05040100u);
+        e0[1] = __builtin_amdgcn_perm(reg[u_][3][j], reg[u_][2][j], 0x05040100u);
+        e1[0] = __builtin_amdgcn_perm(reg[u_][1][j], reg[u_][0][j], 0x07060302u);
+        e1[1] = __builtin_amdgcn_perm(reg[u_][3][j], reg[u_][2][j], 0x07060302u);
         *(u32x2*)(Vt + (ch * 8 + 2 * j) * SM::VST + r0 * 2) = e0;
         *(u32x2*)(Vt + (ch * 8 + 2 * j + 1) * SM::VST + r0 * 2) = e1;
       }
     }
   };
+  auto qk_tile = [&](const unsigned char* Ks, f32x16 (&s)[2]) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
+    // the two 32-key chunks are independent accumulation chains: interleave them
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const bf16x8 a = *(const bf16x8*)(Ks + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
+        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s[c], 0, 0, 0);
+      }
+    }
+  };
 
-  // ---- 3. main loop -------------------------------------------------------------------
+  // ---- 4. main loop -------------------------------------------------------------------------
   f32x16 acc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  float m_run = -INFINITY;  // running max (log2 domain), same in both half-waves
+  float m_run = -INFINITY;  // running reference max (log2 domain), same in both half-waves
   float l_run = 0.f;        // this lane's partial row sum
-  const int q_idx = q_row0 + l32;
 
-  if (T > 0) load_tile(0);
-  for (int t = 0; t < T; ++t) {
+  if (T > 0) {
+    __syncthreads();  // tile descriptors visible
+    u32x4 kreg[PER][4], vreg[PER][4];
+    f32x16 s_a[2], s_b[2];
+    const int Tm1 = T - 1;
+    auto clampt = [&](int t) __attribute__((always_inline)) { return t < Tm1 ? t : Tm1; };
+    // prologue: K(0), V(0) -> LDS; S(0); K(1) -> LDS; {K(2), V(1)} in flight
+    load_rows(0, kb0, P_k_sl, P_kp, kreg, false);
+    load_rows(0, vb0, P_v_sl, P_vp, vreg, true);
+    store_k(Kbuf(0), kreg);
+    store_vt(Vbuf(0), vreg);
+    load_rows(clampt(1), kb0, P_k_sl, P_kp, kreg, false);
     __syncthreads();
-    store_tile();
+    qk_tile(Kbuf(0), s_a);
+    store_k(Kbuf(1), kreg);
+    load_rows(clampt(2), kb0, P_k_sl, P_kp, kreg, false);
+    load_rows(clampt(1), vb0, P_v_sl, P_vp, vreg, true);
     __syncthreads();
-    const int lv = tile_level(t);
-    const int lt = t - toff[lv];
-    const int sbs_log2 = p.bn_log2 - lv;
-    const int c_lv = lv == 0 ? cnt[0] : (lv == 1 ? cnt[1] : (lv == 2 ? cnt[2] : cnt[3]));
-    const int io_lv = lv == 0 ? ioff[0] : (lv == 1 ? ioff[1] : (lv == 2 ? ioff[2] : ioff[3]));
-    if (t + 1 < T) load_tile(t + 1);
 
-    // valid slots form a prefix of the tile
-    int nvalid = TK;
-    int last_blk;
-    if (sbs_log2 >= 6) {
-      last_blk = ids[io_lv + (lt >> (sbs_log2 - 6))];
-      if (lv == 0) {
-        const int rem = p.L - ((last_blk << sbs_log2) + ((lt & ((1 << (sbs_log2 - 6)) - 1)) << 6));
-        nvalid = rem < TK ? rem : TK;
-      }
-    } else {
-      const int bpt = 1 << (6 - sbs_log2);
-      int nb = c_lv - lt * bpt;
-      nb = nb < bpt ? nb : bpt;
-      last_blk = ids[io_lv + lt * bpt + nb - 1];
-      nvalid = nb << sbs_log2;
-      if (lv == 0) {
-        const int rem = p.L - (last_blk << sbs_log2);
-        if (rem < (1 << sbs_log2)) nvalid -= (1 << sbs_log2) - rem;
-      }
-    }
-    const bool diag = p.causal && ((((int64_t)last_blk + 1) << p.bn_log2) - 1 > (int64_t)I * p.bm);
-    const bool masked = diag || nvalid < TK;
-    const int nchunk = nvalid > 32 ? 2 : 1;
+    auto step = [&](int t, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2]) {
+      // invariant: s_cur = raw S^T of tile t; Kbuf((t+1)&1) = K(t+1); Vbuf(t&1) = V(t);
+      //            kreg = K(t+2), vreg = V(t+1) (loads in flight)
+      const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
+      const int lv = d & 3;
+      store_k(Kbuf(t), kreg);
+      store_vt(Vbuf(t + 1), vreg);
+      load_rows(clampt(t + 3), kb0, P_k_sl, P_kp, kreg, false);
+      load_rows(clampt(t + 2), vb0, P_v_sl, P_vp, vreg, true);
 
-    // S^T chunks: 32 keys x 32 queries each
-    f32x16 s[2];
+      if (d & 4) {  // partly empty tile and/or causal diagonal: mask individual keys
+        const TileRef r = tile_ref(t);
+        const int nvalid = (int)((d >> 3) & 127);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
-      if (c < nchunk) {
-        const unsigned char* kr = Ks + (c * 32 + l32) * SM::KST + hh * 16;
+          for (int g = 0; g < 4; ++g) {
+            const int r0 = c * 32 + g * 8 + hh * 4;
+            int src0 = -1;
+            if (r0 < nvalid) src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          const bf16x8 a = *(const bf16x8*)(kr + kk * 32);
-          s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s[c], 0, 0, 0);
-        }
-      }
-    }
-
-    if (masked) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int r0 = c * 32 + g * 8 + hh * 4;
-          int src0 = -1;
-          if (r0 < nvalid) src0 = slot_src(lv, lt, r0, sbs_log2, c_lv, ids + io_lv, p.L);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            bool ok = src0 >= 0 && (r0 + e) < nvalid;
-            if (ok && p.causal) ok = (((int64_t)(src0 + e) + 1) << lv) - 1 <= (int64_t)q_idx;
-            if (!ok) s[c][g * 4 + e] = -INFINITY;
+            for (int e = 0; e < 4; ++e) {
+              const bool in_tile = src0 >= 0 && (r0 + e) < nvalid;
+              // causal: a pooled key is visible once its last constituent token is
+              const bool visible = !P_causal || ((((int64_t)(src0 + e) + 1) << lv) - 1 <= (int64_t)q_idx);
+              const float sv = s_cur[c][g * 4 + e];
+              s_cur[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
+            }
           }
-        }
-    }
+      }
 
-    // online softmax over this tile (per query column = per lane, both half-waves)
-    float mx = s[0][0];
+      // next tile's scores on the MFMA pipe while this tile's softmax runs on the VALU
+      __builtin_amdgcn_s_setprio(1);
+      qk_tile(Kbuf(t + 1), s_nxt);
+      __builtin_amdgcn_s_setprio(0);
+
+      // online softmax of tile t (per query column = per lane, both half-waves)
+      float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
 #pragma unroll
-    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[0][i]);
-    if (nchunk == 2) {
+      for (int i = 1; i < 16; ++i) mx = max3f(mx, s_cur[0][i], s_cur[1][i]);
+      mx = fmaxf(mx, shfl_xor32(mx));
+      const float bias = (float)lv;
+      const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
+      // raise the reference max only when it lags by more than the threshold (or is still -inf)
+      float m_new = (m_cand - m_run > LAZY_THRESHOLD) ? m_cand : m_run;
+      m_new = (m_run == -INFINITY) ? m_cand : m_new;
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that still see no key
+      const float alpha = fast_exp2(m_run - m_use);
+      const float nb = bias - m_use;
+      float lsum0 = 0.f, lsum1 = 0.f;
+      uint32_t pk[2][8];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][i]);
-    }
-    mx = fmaxf(mx, shfl_xor32(mx));
-    const float bias = (float)lv;
-    float m_new = fmaxf(m_run, mx * p.scale_log2 + bias);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that still see no key
-    const float alpha = fast_exp2(m_run - m_use);
-    const float nb = bias - m_use;
-    float lsum = 0.f;
-    uint32_t pk[2][8];
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      if (c < nchunk) {
+      for (int c = 0; c < 2; ++c) {
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-          const float p0 = fast_exp2(__builtin_fmaf(s[c][i], p.scale_log2, nb));
-          const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], p.scale_log2, nb));
-          lsum += p0 + p1;
+          const float p0 = fast_exp2(__builtin_fmaf(s_cur[c][i], P_scale_log2, nb));
+          const float p1 = fast_exp2(__builtin_fmaf(s_cur[c][i + 1], P_scale_log2, nb));
+          lsum0 += p0;
+          lsum1 += p1;
           pk[c][i >> 1] = pack_bf16x2(p0, p1);
         }
       }
-    }
-    l_run = l_run * alpha + lsum;
-    m_run = m_new;
+      l_run = l_run * alpha + (lsum0 + lsum1);
+      m_run = m_new;
 
-    if (__any(alpha != 1.0f)) {
+      if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
-    }
+          for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+      }
 
-    // O^T += V^T P^T : per 16-key group g, A = V^T[32 d][16 keys], B = P^T[16 keys][32 q]
+      // O^T += V^T P^T : per 16-key group g, A = V^T[32 d][16 keys], B = P^T[16 keys][32 q]
+      const unsigned char* Vt = Vbuf(t);
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      if (c < nchunk) {
+      for (int c = 0; c < 2; ++c) {
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
           u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
@@ -374,16 +432,23 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
           }
         }
       }
+      __builtin_amdgcn_s_setprio(0);
+      __syncthreads();
+    };
+    // two tiles per trip: the S^T buffers swap roles without being copied
+    for (int t = 0; t < T; t += 2) {
+      step(t, s_a, s_b);
+      if (t + 1 < T) step(t + 1, s_b, s_a);
     }
   }
 
-  // ---- 4. epilogue --------------------------------------------------------------------
+  // ---- 5. epilogue --------------------------------------------------------------------------
   float l_tot = l_run + shfl_xor32(l_run);
   const float l_safe = fmaxf(l_tot, 1e-8f);
   const float inv = 1.0f / l_safe;
-  if (p.lse != nullptr && hh == 0 && q_idx < p.L) {
+  if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
     // natural-log domain: m*ln2 + ln(max(l, 1e-8))
-    p.lse[((int64_t)b * p.Hq + h) * p.L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
   }
   __syncthreads();  // everyone is done with the last K/V tile
   unsigned char* Os = smem;
@@ -401,14 +466,15 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_kernel(FwdParams p) {
   for (int u = tid; u < BM * CH; u += NT) {
     const int r = u / CH, ch = u % CH;
     const int row = I * BM + r;
-    if (row < p.L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * SM::OST + ch * 16);
+    if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * SM::OST + ch * 16);
   }
 }
 
 template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   using SM = Smem<D>;
-  size_t shmem = (size_t)SM::tile_region(NW * 32) + (size_t)Nk * 2;
+  size_t shmem = (size_t)SM::TILE_BYTES + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
+  if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
   if (shmem > 48 * 1024) {
     if (hipFuncSetAttribute((const void*)psa_fwd_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
       return PSA_ERR_LAUNCH;
@@ -427,6 +493,7 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0, PSA_ERR_ARG, "psa_fwd: B, H, L must be positive");
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_fwd: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
+  PSA_REQUIRE(sm_scale > 0.f, PSA_ERR_ARG, "psa_fwd: sm_scale must be positive");
   PSA_REQUIRE(D == 64 || D == 128, PSA_ERR_UNSUPPORTED, "psa_fwd: head dim %d not in {64, 128}", D);
   PSA_REQUIRE(block_m == 64 || block_m == 128, PSA_ERR_UNSUPPORTED, "psa_fwd: block_m=%d not in {64, 128}", block_m);
   PSA_REQUIRE(block_n == 32 || block_n == 64 || block_n == 128, PSA_ERR_UNSUPPORTED, "psa_fwd: block_n=%d not in {32, 64, 128}", block_n);
@@ -434,6 +501,8 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   for (int i = 0; i < 4; ++i)
     PSA_REQUIRE(((uintptr_t)ts[i]->ptr % 16 == 0) && ts[i]->stride_b % 8 == 0 && ts[i]->stride_h % 8 == 0 && ts[i]->stride_l % 8 == 0,
                 PSA_ERR_UNSUPPORTED, "psa_fwd: tensors must be 16-byte aligned with strides that are multiples of 8 elements");
+  PSA_REQUIRE((int64_t)L * k.stride_l * 2 < (1ll << 32) && (int64_t)L * v.stride_l * 2 < (1ll << 32), PSA_ERR_UNSUPPORTED,
+              "psa_fwd: one (batch, head) slice of K/V must span less than 4 GiB");
   const int Mq = (L + block_m - 1) / block_m, Nk = (L + block_n - 1) / block_n;
   PSA_REQUIRE(Nk <= 65535, PSA_ERR_UNSUPPORTED, "psa_fwd: more than 65535 kv-blocks");
   const int64_t total = (int64_t)B * Hq * Mq;
@@ -453,11 +522,13 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.causal = causal ? 1 : 0;
   p.total_wg = (int)total;
   p.wg_chunk = (int)((total + 7) / 8);
+  // worst case: every kv-block at level 1, plus one partly filled tile per pooled level
+  p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
   int rc;
   if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
   else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);
   else if (block_m == 128) rc = launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
   else rc = launch_fwd<64, 2>(p, Nk, (hipStream_t)stream);
-  PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: launch configuration failed (LDS)");
+  PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");
   return psa_check_launch("psa_fwd");
 }
