@@ -61,6 +61,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention comparison legs (keeps kernel profiles clean)")
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -137,8 +138,10 @@ def main():
     t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
     out_buf = torch.empty_like(q)
     t_fwd_med, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf), it)
-    t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
-    t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
+    t_dense = t_sdpa = None
+    if not args.no_dense:
+        t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
+        t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
 
     pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
@@ -210,9 +213,10 @@ def main():
         "pool_gbs": round(pool_bytes / (t_pool * 1e-3) / 1e9, 1),
         "pool_pct_hbm": round(100 * pool_bytes / (t_pool * 1e-3) / 1e9 / PEAK_HBM_GBS, 2),
         "estimate_tflops": round(est_flops / (t_est * 1e-3) / 1e12, 2),
-        "dense_fa": {"own_kernel_ms": round(t_dense, 3), "own_kernel_tflops": round(dense_flops / (t_dense * 1e-3) / 1e12, 1),
-                     "torch_sdpa_ms": round(t_sdpa, 3), "layer_speedup_vs_own_dense": round(t_dense / ms_step, 2),
-                     "layer_speedup_vs_sdpa": round(t_sdpa / ms_step, 2)},
+        "dense_fa": None if t_dense is None else {
+            "own_kernel_ms": round(t_dense, 3), "own_kernel_tflops": round(dense_flops / (t_dense * 1e-3) / 1e12, 1),
+            "torch_sdpa_ms": round(t_sdpa, 3), "layer_speedup_vs_own_dense": round(t_dense / ms_step, 2),
+            "layer_speedup_vs_sdpa": round(t_sdpa / ms_step, 2)},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

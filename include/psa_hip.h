@@ -7,7 +7,8 @@
  * and re-exposes the reference's names and signatures.
  *
  * Conventions
- *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated or freed here;
+ *   - every pointer is a DEVICE pointer owned by the caller (the small item_* configuration arrays of
+ *     psa_level_map are the one exception: they are read on the host); nothing is allocated or freed here;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*), no host synchronisation;
  *   - return value 0 = ok, negative = error (see PSA_ERR_*); psa_last_error() gives a
  *     thread-local human-readable message for the last failing call on this thread;
@@ -64,17 +65,22 @@ int64_t psa_pool_level_offset(int B, int Hkv, int L, int D, int block_n, int lev
 int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_pool,
                 int B, int Hkv, int L, int D, int block_n, psa_stream_t stream);
 
+/* Bytes of scratch psa_estimate_sampled needs (the per-row key-group maxima in fp32). */
+int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, int block_m, int block_n,
+                                     int keep_m, int keep_n);
+
 /* Sampled block-importance estimate.  Row r of the sampled Q is source row
  * min((r/keep_m)*block_m + off_q[b,h,r%keep_m], Lq-1) (off_q == NULL: offsets 0..keep_m-1, i.e. the
  * input is already sampled when block_m == keep_m); rows past the last sampled row replicate it up to
  * a multiple of 64, as the reference pads.  Same for K with off_k [B, Hkv, keep_n].
  * scores [B, Hq, out_rows, out_cols] fp32 = rows normalised by the sum over ALL key groups
- * (including the padding groups), cropped to out_rows x out_cols.
+ * (including the padding groups), cropped to out_rows x out_cols.  `workspace` is caller-allocated
+ * device memory of psa_estimate_workspace_bytes(...) bytes; its contents are overwritten.
  * Replaces _random_sample_tokens' gather + attn_with_pooling_optimized:
  *   reference src/psa_triton/attention.py:116-137,178-223,
  *   src/psa_triton/kernels/attn_pooling_kernel.py:12-116,119-282,285-451. */
 int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k,
-                         float* scores, int B, int Hq, int Hkv, int Lq, int Lk, int D,
+                         float* scores, void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D,
                          int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
                          int out_rows, int out_cols, psa_stream_t stream);
 

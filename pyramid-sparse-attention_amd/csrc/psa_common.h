@@ -56,6 +56,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// v_max3_f32.  The compiler does not track hazards for inline assembly: never feed it a value that an
+// MFMA instruction has just produced (the required wait states are only inserted for instructions
+// the compiler knows); values that went through another VALU op, or are a loop iteration old, are fine.
 __device__ __forceinline__ float max3f(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));

@@ -1,34 +1,35 @@
-// Sampled block-importance estimator: a dense bf16 MFMA contraction of the sampled query rows with
-// the sampled key rows, with the reference's max-pooling epilogue fused in, so neither the sampled
-// tensors nor the per-row group maxima ever touch HBM.
+// Sampled block-importance estimator.
 //
 //   R[r, j]  = max_{c in key group j} (q_r . k_c) * scale * log2(e)
 //   m[r]     = max_j R[r, j]
 //   Po[i, j] = max_{r in query group i} exp2(R[r, j] - m[r]);   Po[i, :] /= sum_j Po[i, j]
 //
-// One workgroup = NW waves x 32 sampled query rows; all waves share the K tile (64 sampled keys,
-// gathered straight from the un-sampled K through the per-head offset table).  As in the forward
-// kernel the transposed product S^T = K Q^T is computed, so that a lane holds 16 keys of one query
-// row and a key-group maximum is an in-lane reduction plus one half-wave exchange.  R for the
-// workgroup's rows stays in LDS (fp32, [key group][33]) until the row maxima are final.
-//
-// Roofline: MFMA-bound (2 * Ms * Ns * D flops against ~(Ms + Ns) * D * 2 bytes).
+// Kernel 1 (MFMA-bound, 2*Ms*Ns*D flops): a dense bf16 contraction of the sampled query rows with the
+// sampled key rows, both gathered straight from the un-sampled Q / K through the per-head offset
+// tables.  One workgroup = NW waves x 32 sampled query rows; the waves share K tiles of 64 sampled
+// keys, double-buffered in LDS (one barrier per tile, global loads two tiles ahead).  As in the
+// forward kernel the transposed product S^T = K Q^T is computed, so a lane holds 16 keys of one query
+// row and a key-group maximum is an in-lane reduction plus one half-wave exchange.  The group maxima
+// go to an fp32 workspace laid out [key group][query row], i.e. 128-byte coalesced stores.
+// Kernel 2 (HBM-bound, reads the workspace once): per (query group, key group) the maximum over the
+// group's rows of R - m, exp2, row sum in a fixed order, normalisation.
 #include "psa_common.h"
 
 namespace {
 
 constexpr int TK = 64;
-constexpr int RST = 33;  // floats per key-group row of the R buffer (32 + 1 pad)
 
 struct EstParams {
   const bf16_t *q, *k;
   int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl;
   const int32_t *off_q, *off_k;
+  float* rt;   // workspace: R^T [B*Hq][n_d][Ms_pad]
+  float* mrow; // workspace: m [B*Hq][Ms_pad]
   float* scores;
   int Hq, Hkv, Lq, Lk;
   int bm, bn, keep_m_log2, keep_n_log2;
-  int Ms, Ns, Ns_pad;  // real sampled rows / keys, padded key count (multiple of 64)
-  int n_d;             // key groups incl. padding groups
+  int Ms, Ns, Ms_pad, Ns_pad;  // real sampled rows / keys, padded counts (multiples of 64)
+  int n_d;                     // key groups incl. padding groups
   int out_rows, out_cols;
   float qk_scale;
 };
@@ -41,18 +42,16 @@ __device__ __forceinline__ int sampled_src(int r, int n_real, int keep_log2, int
 }
 
 template <int D, int NW>
-__global__ __launch_bounds__(NW * 64) void psa_estimate_kernel(EstParams p) {
+__global__ __launch_bounds__(NW * 64, 2) void psa_est_gemm_kernel(EstParams p) {
   constexpr int NT = NW * 64;
   constexpr int CH = D / 8;
   constexpr int UNITS = 16 * CH;
   constexpr int PER = (UNITS + NT - 1) / NT;
   constexpr int KK = D / 16;
   constexpr int KST = D * 2 + 16;
+  constexpr int K_BYTES = TK * KST;
 
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* Ks = smem;
-  float* Rl = (float*)(smem + TK * KST);  // [NW][n_d][RST]
-  float* ml = Rl + (size_t)NW * p.n_d * RST;  // [NW][32]
+  __shared__ __align__(16) unsigned char smem[2 * K_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
@@ -72,10 +71,24 @@ __global__ __launch_bounds__(NW * 64) void psa_estimate_kernel(EstParams p) {
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
   }
 
-  const bf16_t* kb = p.k + b * p.k_sb + hk * p.k_sh;
+  const char* kb = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  const uint32_t kstrb = (uint32_t)p.k_sl * 2u;
   const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * keep_n : nullptr;
+  // a thread always handles the same in-group positions: tiles are 64 keys and keep_n divides 64
+  int my_off[PER][4];
+#pragma unroll
+  for (int u_ = 0; u_ < PER; ++u_) {
+    const int u = tid + u_ * NT;
+    const int r0 = (u / CH) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = (r0 + i) & (keep_n - 1);
+      my_off[u_][i] = ok ? ok[e] : e;
+    }
+  }
+  const int Ns = p.Ns, Lk = p.Lk, bn = p.bn, kn_log2 = p.keep_n_log2;
   u32x4 kreg[PER][4];
-  auto load_tile = [&](int t) {
+  auto load_tile = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
     for (int u_ = 0; u_ < PER; ++u_) {
       const int u = tid + u_ * NT;
@@ -83,12 +96,20 @@ __global__ __launch_bounds__(NW * 64) void psa_estimate_kernel(EstParams p) {
       const int r0 = (u / CH) * 4, ch = u % CH;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int src = sampled_src(t * TK + r0 + i, p.Ns, p.keep_n_log2, p.bn, ok, p.Lk);
-        kreg[u_][i] = *(const u32x4*)(kb + (int64_t)src * p.k_sl + ch * 8);
+        int r = t * TK + r0 + i;
+        int src;
+        if (r < Ns) {
+          src = (r >> kn_log2) * bn + my_off[u_][i];
+        } else {  // padding keys replicate the last sampled key
+          r = Ns - 1;
+          src = (r >> kn_log2) * bn + (ok ? ok[r & ((1 << kn_log2) - 1)] : (r & ((1 << kn_log2) - 1)));
+        }
+        src = src < Lk ? src : Lk - 1;
+        kreg[u_][i] = *(const u32x4*)(kb + ((uint32_t)src * kstrb + (uint32_t)(ch * 16)));
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](unsigned char* Ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int u_ = 0; u_ < PER; ++u_) {
       const int u = tid + u_ * NT;
@@ -99,102 +120,157 @@ __global__ __launch_bounds__(NW * 64) void psa_estimate_kernel(EstParams p) {
     }
   };
 
-  float* Rw = Rl + (size_t)wave * p.n_d * RST;
-  float m_run = -INFINITY;
   const int T = p.Ns_pad / TK;
   const int gpc_log2 = 5 - p.keep_n_log2;  // key groups per 32-key chunk (1, 2 or 4)
+  float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + row0 + l32;
+  const int64_t rts = p.Ms_pad;
+  float m_run = -INFINITY;
+  const float qk_scale = p.qk_scale;
 
   load_tile(0);
+  store_tile(smem);
+  load_tile(T > 1 ? 1 : 0);
+  __syncthreads();
   for (int t = 0; t < T; ++t) {
-    __syncthreads();
-    store_tile();
-    __syncthreads();
-    if (t + 1 < T) load_tile(t + 1);
+    // invariant: buffer t&1 holds tile t; kreg holds tile t+1 (in flight)
+    store_tile(smem + ((t + 1) & 1) * K_BYTES);
+    load_tile(t + 2 < T ? t + 2 : T - 1);
+    const unsigned char* Ks = smem + (t & 1) * K_BYTES;
+    f32x16 s[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const bf16x8 a = *(const bf16x8*)(Ks + (c * 32 + l32) * KST + hh * 16 + kk * 32);
+        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s[c], 0, 0, 0);
+      }
+    }
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-      f32x16 s;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = 0.f;
-      const unsigned char* kr = Ks + (c * 32 + l32) * KST + hh * 16;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const bf16x8 a = *(const bf16x8*)(kr + kk * 32);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
-      }
       // register i holds key (i/4)*8 + hh*4 + i%4 of this chunk: 8-key octets are registers 4o..4o+3
       float o4[4];
 #pragma unroll
-      for (int o = 0; o < 4; ++o) o4[o] = fmaxf(fmaxf(s[4 * o], s[4 * o + 1]), fmaxf(s[4 * o + 2], s[4 * o + 3]));
+      for (int o = 0; o < 4; ++o) o4[o] = fmaxf(fmaxf(s[c][4 * o], s[c][4 * o + 1]), fmaxf(s[c][4 * o + 2], s[c][4 * o + 3]));
       const int jbase = (t * 2 + c) << gpc_log2;
       if (gpc_log2 == 0) {
         float v = fmaxf(fmaxf(o4[0], o4[1]), fmaxf(o4[2], o4[3]));
-        v = fmaxf(v, shfl_xor32(v)) * p.qk_scale;
+        v = fmaxf(v, shfl_xor32(v)) * qk_scale;
         m_run = fmaxf(m_run, v);
-        if (hh == 0) Rw[jbase * RST + l32] = v;
+        if (hh == 0) rt[(int64_t)jbase * rts] = v;
       } else if (gpc_log2 == 1) {
         float v0 = fmaxf(o4[0], o4[1]), v1 = fmaxf(o4[2], o4[3]);
-        v0 = fmaxf(v0, shfl_xor32(v0)) * p.qk_scale;
-        v1 = fmaxf(v1, shfl_xor32(v1)) * p.qk_scale;
+        v0 = fmaxf(v0, shfl_xor32(v0)) * qk_scale;
+        v1 = fmaxf(v1, shfl_xor32(v1)) * qk_scale;
         m_run = fmaxf(m_run, fmaxf(v0, v1));
-        if (hh == 0) {
-          Rw[jbase * RST + l32] = v0;
-          Rw[(jbase + 1) * RST + l32] = v1;
-        }
+        rt[(int64_t)(jbase + hh) * rts] = hh ? v1 : v0;
       } else {
 #pragma unroll
         for (int o = 0; o < 4; ++o) {
-          const float v = fmaxf(o4[o], shfl_xor32(o4[o])) * p.qk_scale;
+          const float v = fmaxf(o4[o], shfl_xor32(o4[o])) * qk_scale;
           m_run = fmaxf(m_run, v);
-          if (hh == 0) Rw[(jbase + o) * RST + l32] = v;
+          if ((o & 1) == hh) rt[(int64_t)(jbase + o) * rts] = v;
         }
       }
     }
+    __syncthreads();
   }
-  if (hh == 0) ml[wave * 32 + l32] = m_run;
-  __syncthreads();
+  if (hh == 0) p.mrow[(int64_t)bh * p.Ms_pad + row0 + l32] = m_run;
+}
 
-  // phase 2: per query group, Po[j] = exp2(max_r (R[r][j] - m[r])), normalised by the sum over ALL n_d
-  const float* mw = ml + wave * 32;
-  const int groups = 32 >> p.keep_m_log2;
-  for (int g = 0; g < groups; ++g) {
-    const int grow = ((row0 + g * keep_m) >> p.keep_m_log2);
-    const int r_lo = g * keep_m;
-    float part = 0.f;
-    for (int j = lane; j < p.n_d; j += 64) {
-      float v = -INFINITY;
-      for (int r = 0; r < keep_m; ++r) v = fmaxf(v, Rw[j * RST + r_lo + r] - mw[r_lo + r]);
-      const float e = fast_exp2(v);
-      Rw[j * RST + r_lo] = e;
-      part += e;
+// one workgroup per (b, h, query group): Po[i, :] from R^T and m
+__global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
+  __shared__ float s_m[32];
+  __shared__ float s_part[4];
+  __shared__ float s_total;
+  const int i = blockIdx.x, bh = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int keep_m = 1 << p.keep_m_log2;
+  const int r0 = i * keep_m;
+  if (tid < keep_m) s_m[tid] = p.mrow[(int64_t)bh * p.Ms_pad + r0 + tid];
+  __syncthreads();
+  const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0;
+  // every thread owns key groups tid, tid+256, ...; their values are kept for the normalisation pass
+  float part = 0.f;
+  float keep[8];
+  int nk = 0;
+  for (int j = tid; j < p.n_d; j += 256, ++nk) {
+    const float* src = rt + (int64_t)j * p.Ms_pad;
+    float v = -INFINITY;
+    for (int r = 0; r < keep_m; r += 4) {
+      const f32x4 x = *(const f32x4*)(src + r);
+      v = fmaxf(v, fmaxf(fmaxf(x[0] - s_m[r], x[1] - s_m[r + 1]), fmaxf(x[2] - s_m[r + 2], x[3] - s_m[r + 3])));
     }
+    const float e = fast_exp2(v);
+    if (nk < 8) keep[nk] = e;
+    part += e;
+  }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-    if (grow < p.out_rows) {
-      float* dst = p.scores + ((int64_t)bh * p.out_rows + grow) * p.out_cols;
-      for (int j = lane; j < p.out_cols; j += 64) dst[j] = Rw[j * RST + r_lo] / part;
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+  if ((tid & 63) == 0) s_part[tid >> 6] = part;
+  __syncthreads();
+  if (tid == 0) s_total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+  __syncthreads();
+  const float total = s_total;
+  float* dst = p.scores + ((int64_t)bh * p.out_rows + i) * p.out_cols;
+  nk = 0;
+  for (int j = tid; j < p.n_d; j += 256, ++nk) {
+    float e;
+    if (nk < 8) {
+      e = keep[nk];
+    } else {  // very wide rows: recompute
+      const float* src = rt + (int64_t)j * p.Ms_pad;
+      float v = -INFINITY;
+      for (int r = 0; r < keep_m; ++r) v = fmaxf(v, src[r] - s_m[r]);
+      e = fast_exp2(v);
     }
+    if (j < p.out_cols) dst[j] = e / total;
   }
 }
 
-template <int D, int NW>
-int launch_est(const EstParams& p, int B, int q_rows_needed, hipStream_t stream) {
-  size_t shmem = (size_t)TK * (D * 2 + 16) + ((size_t)NW * p.n_d * RST + NW * 32) * sizeof(float);
-  if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-  if (shmem > 48 * 1024) {
-    if (hipFuncSetAttribute((const void*)psa_estimate_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-      return PSA_ERR_LAUNCH;
-  }
-  dim3 grid((unsigned)((q_rows_needed + NW * 32 - 1) / (NW * 32)), (unsigned)(B * p.Hq));
-  hipLaunchKernelGGL((psa_estimate_kernel<D, NW>), grid, dim3(NW * 64), shmem, stream, p);
-  return PSA_OK;
+template <int D>
+int launch_est(const EstParams& p, int B, hipStream_t stream) {
+  constexpr int NW = 4;
+  const int rows_needed = p.out_rows << p.keep_m_log2;
+  dim3 grid((unsigned)((rows_needed + NW * 32 - 1) / (NW * 32)), (unsigned)(B * p.Hq));
+  hipLaunchKernelGGL((psa_est_gemm_kernel<D, NW>), grid, dim3(NW * 64), 0, stream, p);
+  const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
+  if (rc != PSA_OK) return rc;
+  hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), 0, stream, p);
+  return psa_check_launch("psa_estimate_sampled (reduction)");
+}
+
+struct EstGeom {
+  int Ms, Ns, Ms_pad, Ns_pad, m_d, n_d;
+};
+EstGeom est_geom(int Lq, int Lk, int block_m, int block_n, int keep_m, int keep_n) {
+  EstGeom g;
+  const int Mq = (Lq + block_m - 1) / block_m, Nk = (Lk + block_n - 1) / block_n;
+  g.Ms = Mq * keep_m;
+  g.Ns = Nk * keep_n;
+  // the GEMM kernel works on 128 query rows per workgroup; the reference pads to 64
+  g.Ms_pad = (g.Ms + 127) / 128 * 128;
+  g.Ns_pad = (g.Ns + 63) / 64 * 64;
+  g.m_d = ((g.Ms + 63) / 64 * 64) / keep_m;
+  g.n_d = g.Ns_pad / keep_n;
+  return g;
 }
 
 }  // namespace
 
+extern "C" int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, int block_m, int block_n, int keep_m, int keep_n) {
+  if (B <= 0 || Hq <= 0 || Lq <= 0 || Lk <= 0 || block_m <= 0 || block_n <= 0 || keep_m <= 0 || keep_n <= 0) return 0;
+  const EstGeom g = est_geom(Lq, Lk, block_m, block_n, keep_m, keep_n);
+  return (int64_t)B * Hq * ((int64_t)g.n_d + 1) * g.Ms_pad * (int64_t)sizeof(float);
+}
+
 extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
-                                    int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n, int keep_m,
-                                    int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
-  PSA_REQUIRE(q.ptr && k.ptr && scores, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
+                                    void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
+                                    int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
+  PSA_REQUIRE(q.ptr && k.ptr && scores && workspace, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Lq > 0 && Lk > 0, PSA_ERR_ARG, "psa_estimate_sampled: sizes must be positive");
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_estimate_sampled: Hq must be a multiple of Hkv");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: B*Hq too large");
@@ -205,6 +281,9 @@ extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t*
   PSA_REQUIRE(((uintptr_t)q.ptr % 16 == 0) && ((uintptr_t)k.ptr % 16 == 0) && q.stride_l % 8 == 0 && k.stride_l % 8 == 0 &&
                   q.stride_h % 8 == 0 && k.stride_h % 8 == 0 && q.stride_b % 8 == 0 && k.stride_b % 8 == 0,
               PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: tensors must be 16-byte aligned with strides multiple of 8");
+  PSA_REQUIRE((int64_t)Lk * k.stride_l * 2 < (1ll << 32), PSA_ERR_UNSUPPORTED,
+              "psa_estimate_sampled: one (batch, head) slice of K must span less than 4 GiB");
+  const EstGeom g = est_geom(Lq, Lk, block_m, block_n, keep_m, keep_n);
   EstParams p;
   p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr;
   p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sl = q.stride_l;
@@ -212,28 +291,12 @@ extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t*
   p.off_q = off_q; p.off_k = off_k; p.scores = scores;
   p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.bm = block_m; p.bn = block_n;
   p.keep_m_log2 = psa_ilog2(keep_m); p.keep_n_log2 = psa_ilog2(keep_n);
-  const int Mq = (Lq + block_m - 1) / block_m, Nk = (Lk + block_n - 1) / block_n;
-  p.Ms = Mq * keep_m; p.Ns = Nk * keep_n;
-  const int Ms_pad = (p.Ms + 63) / 64 * 64;
-  p.Ns_pad = (p.Ns + 63) / 64 * 64;
-  p.n_d = p.Ns_pad / keep_n;
-  const int m_d = Ms_pad / keep_m;
-  PSA_REQUIRE(out_rows > 0 && out_rows <= m_d && out_cols > 0 && out_cols <= p.n_d, PSA_ERR_ARG,
-              "psa_estimate_sampled: out_rows/out_cols exceed %d x %d", m_d, p.n_d);
+  p.Ms = g.Ms; p.Ns = g.Ns; p.Ms_pad = g.Ms_pad; p.Ns_pad = g.Ns_pad; p.n_d = g.n_d;
+  PSA_REQUIRE(out_rows > 0 && out_rows <= g.m_d && out_cols > 0 && out_cols <= g.n_d, PSA_ERR_ARG,
+              "psa_estimate_sampled: out_rows/out_cols exceed %d x %d", g.m_d, g.n_d);
   p.out_rows = out_rows; p.out_cols = out_cols;
   p.qk_scale = sm_scale * 1.44269504f;
-  const int rows_needed = out_rows * keep_m;
-  // waves per workgroup: as many as the R buffer lets fit in LDS
-  const size_t kt = (size_t)TK * (D * 2 + 16);
-  int nw = 4;
-  while (nw > 1 && kt + ((size_t)nw * p.n_d * RST + nw * 32) * 4 > 160 * 1024) nw >>= 1;
-  int rc;
-  if (D == 128) rc = nw == 4 ? launch_est<128, 4>(p, B, rows_needed, (hipStream_t)stream)
-                   : nw == 2 ? launch_est<128, 2>(p, B, rows_needed, (hipStream_t)stream)
-                             : launch_est<128, 1>(p, B, rows_needed, (hipStream_t)stream);
-  else rc = nw == 4 ? launch_est<64, 4>(p, B, rows_needed, (hipStream_t)stream)
-            : nw == 2 ? launch_est<64, 2>(p, B, rows_needed, (hipStream_t)stream)
-                      : launch_est<64, 1>(p, B, rows_needed, (hipStream_t)stream);
-  PSA_REQUIRE(rc == PSA_OK, rc, "psa_estimate_sampled: %d key groups do not fit the on-chip score buffer", p.n_d);
-  return psa_check_launch("psa_estimate_sampled");
+  p.rt = (float*)workspace;
+  p.mrow = p.rt + (int64_t)B * Hq * g.n_d * g.Ms_pad;
+  return D == 128 ? launch_est<128>(p, B, (hipStream_t)stream) : launch_est<64>(p, B, (hipStream_t)stream);
 }

@@ -30,9 +30,10 @@ SIGNATURES = {
     "psa_pool_elems": (c_int64, [c_int, c_int, c_int, c_int, c_int]),
     "psa_pool_level_offset": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "psa_pool_kv": (c_int, [Tensor4, Tensor4, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "psa_estimate_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "psa_estimate_sampled": (
         c_int,
-        [Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+        [Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
          c_int, c_float, c_int, c_int, c_void_p],
     ),
     "psa_level_map": (

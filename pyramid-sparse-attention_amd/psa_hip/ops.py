@@ -94,9 +94,10 @@ def estimate_sampled(
         if o is not None and (o.dtype != torch.int32 or tuple(o.shape) != (B, H, keep) or not o.is_contiguous()):
             raise ValueError("sample offsets must be contiguous int32 [B, H, keep]")
     scores = torch.empty(B, Hq, out_rows, out_cols, dtype=torch.float32, device=q.device)
+    ws = torch.empty(lib.psa_estimate_workspace_bytes(B, Hq, Lq, Lk, block_m, block_n, keep_m, keep_n), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
         check(
-            lib.psa_estimate_sampled(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), B, Hq, Hkv, Lq, Lk, D,
+            lib.psa_estimate_sampled(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D,
                                      block_m, block_n, keep_m, keep_n, float(sm_scale), out_rows, out_cols, _stream(q)),
             "psa_estimate_sampled",
         )
