@@ -181,54 +181,38 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_est_gemm_kernel(EstParams p) {
   if (hh == 0) p.mrow[(int64_t)bh * p.Ms_pad + row0 + l32] = m_run;
 }
 
-// one workgroup per (b, h, query group): Po[i, :] from R^T and m
+// one workgroup per (b, h, query group): Po[i, :] from R^T and m.
+// A wave reads 64/keep_m key groups at a time: lane l holds row l % keep_m of key group j0 + l / keep_m,
+// i.e. every keep_m-lane segment reads one contiguous run of the workspace; the maximum over the
+// group's rows is a butterfly inside the segment.
 __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
-  __shared__ float s_m[32];
+  extern __shared__ float s_e[];  // [n_d] un-normalised Po row
   __shared__ float s_part[4];
-  __shared__ float s_total;
   const int i = blockIdx.x, bh = blockIdx.y;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int keep_m = 1 << p.keep_m_log2;
+  const int row = lane & (keep_m - 1), sub = lane >> p.keep_m_log2;
+  const int per_iter = 64 >> p.keep_m_log2;  // key groups per wave iteration
   const int r0 = i * keep_m;
-  if (tid < keep_m) s_m[tid] = p.mrow[(int64_t)bh * p.Ms_pad + r0 + tid];
-  __syncthreads();
-  const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0;
-  // every thread owns key groups tid, tid+256, ...; their values are kept for the normalisation pass
-  float part = 0.f;
-  float keep[8];
-  int nk = 0;
-  for (int j = tid; j < p.n_d; j += 256, ++nk) {
-    const float* src = rt + (int64_t)j * p.Ms_pad;
-    float v = -INFINITY;
-    for (int r = 0; r < keep_m; r += 4) {
-      const f32x4 x = *(const f32x4*)(src + r);
-      v = fmaxf(v, fmaxf(fmaxf(x[0] - s_m[r], x[1] - s_m[r + 1]), fmaxf(x[2] - s_m[r + 2], x[3] - s_m[r + 3])));
-    }
-    const float e = fast_exp2(v);
-    if (nk < 8) keep[nk] = e;
-    part += e;
+  const float m = p.mrow[(int64_t)bh * p.Ms_pad + r0 + row];
+  const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0 + row;
+  for (int j0 = wave * per_iter; j0 < p.n_d; j0 += 4 * per_iter) {
+    const int j = j0 + sub;
+    float v = j < p.n_d ? rt[(int64_t)j * p.Ms_pad] - m : -INFINITY;
+    for (int o = keep_m >> 1; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    if (row == 0 && j < p.n_d) s_e[j] = fast_exp2(v);
   }
+  __syncthreads();
+  // row sum in a fixed order: per-thread strided partials, wave butterfly, four wave partials
+  float part = 0.f;
+  for (int j = tid; j < p.n_d; j += 256) part += s_e[j];
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-  if ((tid & 63) == 0) s_part[tid >> 6] = part;
+  if (lane == 0) s_part[wave] = part;
   __syncthreads();
-  if (tid == 0) s_total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
-  __syncthreads();
-  const float total = s_total;
+  const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
   float* dst = p.scores + ((int64_t)bh * p.out_rows + i) * p.out_cols;
-  nk = 0;
-  for (int j = tid; j < p.n_d; j += 256, ++nk) {
-    float e;
-    if (nk < 8) {
-      e = keep[nk];
-    } else {  // very wide rows: recompute
-      const float* src = rt + (int64_t)j * p.Ms_pad;
-      float v = -INFINITY;
-      for (int r = 0; r < keep_m; ++r) v = fmaxf(v, src[r] - s_m[r]);
-      e = fast_exp2(v);
-    }
-    if (j < p.out_cols) dst[j] = e / total;
-  }
+  for (int j = tid; j < p.out_cols; j += 256) dst[j] = s_e[j] / total;
 }
 
 template <int D>
@@ -239,7 +223,7 @@ int launch_est(const EstParams& p, int B, hipStream_t stream) {
   hipLaunchKernelGGL((psa_est_gemm_kernel<D, NW>), grid, dim3(NW * 64), 0, stream, p);
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
-  hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
   return psa_check_launch("psa_estimate_sampled (reduction)");
 }
 

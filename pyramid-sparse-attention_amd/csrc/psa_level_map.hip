@@ -63,8 +63,19 @@ __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
 
   if (p.mode == PSA_MODE_THRESHOLDBOUND) {
     if (tid == 0) {
+      // strictly sequential fp64 accumulation (the order matters for bit-exactness); the LDS traffic is
+      // batched four values at a time so that only the additions form the dependent chain
       double acc = 0.0;
-      for (int i = 0; i < N; ++i) {
+      int i = 0;
+      for (; i + 4 <= N; i += 4) {
+        const float w0 = sw[i], w1 = sw[i + 1], w2 = sw[i + 2], w3 = sw[i + 3];
+        const double a0 = acc + (double)w0;
+        const double a1 = a0 + (double)w1;
+        const double a2 = a1 + (double)w2;
+        acc = a2 + (double)w3;
+        c32[i] = (float)a0; c32[i + 1] = (float)a1; c32[i + 2] = (float)a2; c32[i + 3] = (float)acc;
+      }
+      for (; i < N; ++i) {
         acc += (double)sw[i];
         c32[i] = (float)acc;
       }
@@ -279,13 +290,12 @@ __global__ __launch_bounds__(256) void psa_density_kernel(const void* map, int m
   const int64_t n = (int64_t)Mq * Nk;
   // counts per level are exact integers; 1/level sums are exact in fp32 up to 2^24/8 blocks
   int c1 = 0, c2 = 0, c4 = 0, c8 = 0;
-  int64_t valid = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 256) {
-    const int r = (int)(i / Nk), c = (int)(i % Nk);
-    if (causal && c > r) continue;
-    ++valid;
-    const int lv = load_map(map, bh * n + i, map_elem);
-    c1 += lv == 1; c2 += lv == 2; c4 += lv == 4; c8 += lv == 8;
+  for (int r = 0; r < Mq; ++r) {
+    const int cend = causal ? (r + 1 < Nk ? r + 1 : Nk) : Nk;
+    for (int c = threadIdx.x; c < cend; c += 256) {
+      const int lv = load_map(map, bh * n + (int64_t)r * Nk + c, map_elem);
+      c1 += lv == 1; c2 += lv == 2; c4 += lv == 4; c8 += lv == 8;
+    }
   }
   float v = (float)c1 + 0.5f * (float)c2 + 0.25f * (float)c4 + 0.125f * (float)c8;
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
