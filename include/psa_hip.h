@@ -127,6 +127,21 @@ int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, con
             int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
             int causal, psa_stream_t stream);
 
+/* Bytes of workspace psa_bwd needs (fp32 dK/dV per pyramid level, delta, lse in log2 units). */
+int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n);
+
+/* Backward of psa_fwd w.r.t. q, k, v (the map carries no gradient).  dq/dk/dv are bf16 views like
+ * q/k/v; workspace is caller-allocated (psa_bwd_workspace_bytes) and is overwritten.
+ * Gradients of pooled keys are spread over their constituent tokens (/level) and the part that
+ * lands on replicate-pad positions is added to the last real token.
+ * Replaces _sparse_attention.backward and its kernels:
+ *   reference src/psa_triton/kernels/psa_kernel_legacy.py:948-1069,1072-1234,1237-1320. */
+int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+            const void* map, int map_elem_bytes, psa_tensor4 out, psa_tensor4 dout, const float* lse,
+            psa_tensor4 dq, psa_tensor4 dk, psa_tensor4 dv, void* workspace,
+            int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
+            int causal, psa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -485,9 +485,12 @@ def psa_attention_dense(
         Vc = Vc.repeat_interleave(n_rep, 1)
     bias = _expanded_keys(levels_k, lmap, block_m, block_n, L, causal).to(dtype)
     S = torch.matmul(q.to(dtype), Kc.transpose(-1, -2)) * sm_scale + bias
-    lse = torch.logsumexp(S, -1)
-    P = torch.exp(S - torch.where(torch.isinf(lse), torch.zeros_like(lse), lse).unsqueeze(-1))
-    P = torch.where(torch.isinf(S) & (S < 0), torch.zeros_like(P), P)
+    # rows without any key: output 0, lse -inf, and (under autograd) zero gradient instead of NaN
+    row_ok = (S > float("-inf")).any(-1, keepdim=True)
+    S_safe = torch.where(row_ok, S, torch.zeros_like(S))
+    lse_safe = torch.logsumexp(S_safe, -1, keepdim=True)
+    P = torch.exp(S_safe - lse_safe) * row_ok.to(dtype)
+    lse = torch.where(row_ok, lse_safe, torch.full_like(lse_safe, float("-inf"))).squeeze(-1)
     out = torch.matmul(P, Vc)
     return out, lse
 

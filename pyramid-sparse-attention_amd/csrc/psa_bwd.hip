@@ -1,0 +1,734 @@
+// Backward of the pyramid sparse attention w.r.t. Q, K, V.
+//
+//   delta_i = sum_d O_id dO_id
+//   p_it    = exp2(scale*log2e * q_i.K_l[t] + log2(l) - lse_i*log2e)     (one value per retained pooled key)
+//   dV_l[t] += sum_i p_it dO_i          dP_it = dO_i . V_l[t]          dS_it = p_it (dP_it - delta_i)
+//   dQ_i    += scale sum_t dS_it K_l[t]                                dK_l[t] += scale sum_i dS_it q_i
+//   dK[n]    = dK_1[n] + sum_{l=2,4,8} dK_l[n/l] / l, the part of replicate-pad rows n >= L added to row L-1
+//
+// Four kernels:
+//   psa_bwd_delta_kernel   HBM-bound: delta and lse in log2 units (rows without keys get +inf so p = 0)
+//   psa_bwd_dq_kernel      MFMA-bound row walk: the forward's tile schedule; per tile S^T = K Q^T,
+//                          dP^T = V dO^T, dQ^T += K^T dS^T on bf16 MFMA, operands pooled K/V read directly
+//   psa_bwd_dkdv_kernel    MFMA-bound column walk: one workgroup per (kv head, kv-block, level slot) keeps its
+//                          <= 64 pooled keys in registers and streams the q-blocks that retain this block at
+//                          this level; dK_l, dV_l go to an fp32 workspace (every row written exactly once)
+//   psa_bwd_unpool_kernel  HBM-bound: sums the levels, spreads pooled gradients, folds the pad tail, -> bf16
+#include "psa_tiles.h"
+
+namespace {
+
+using namespace psa_tiles;
+
+struct BwdParams {
+  const bf16_t *q, *k, *v, *o, *dout;
+  int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, o_sb, o_sh, o_sl, do_sb, do_sh, do_sl;
+  bf16_t *dq, *dk, *dv;
+  int64_t dq_sb, dq_sh, dq_sl, dk_sb, dk_sh, dk_sl, dv_sb, dv_sh, dv_sl;
+  const bf16_t *kp, *vp;
+  const void* map;
+  int map_elem;
+  const float* lse;
+  float *delta, *lse2;  // workspace [B*Hq*L] each
+  float *wk, *wv;       // workspace: per-level fp32 dK / dV, levels back to back: [BHkv, npad >> lv, D]
+  int B, Hq, Hkv, L, Mq, Nk, bn_log2, bm;
+  int64_t npad;
+  float scale, scale_log2;
+  int causal;
+  int max_tiles;
+};
+
+// ------------------------------------------------------------------------------------------------------
+// delta and log2-domain lse
+// ------------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
+  constexpr int LPR = D / 8;  // lanes per row
+  const int bh = blockIdx.y, b = bh / p.Hq, h = bh % p.Hq;
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+  const int c = threadIdx.x % LPR;
+  float acc = 0.f;
+  if (row < p.L) {
+    const u32x4 ow = *(const u32x4*)(p.o + b * p.o_sb + h * p.o_sh + row * p.o_sl + c * 8);
+    const u32x4 dw = *(const u32x4*)(p.dout + b * p.do_sb + h * p.do_sh + row * p.do_sl + c * 8);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc += bf16_bits_to_f32(ow[j] & 0xffffu) * bf16_bits_to_f32(dw[j] & 0xffffu);
+      acc += __builtin_bit_cast(float, ow[j] & 0xffff0000u) * __builtin_bit_cast(float, dw[j] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (c == 0 && row < p.L) {
+    const float l = p.lse[(int64_t)bh * p.L + row];
+    p.delta[(int64_t)bh * p.L + row] = acc;
+    // rows that saw no key have lse = -inf and zero gradient: +inf makes every p vanish
+    p.lse2[(int64_t)bh * p.L + row] = (l == -INFINITY) ? INFINITY : l * 1.4426950408889634f;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------
+// dQ: row walk
+// ------------------------------------------------------------------------------------------------------
+template <int D>
+struct DqSmem {
+  static constexpr int KST = D * 2 + 16;  // bytes per [key][d] row
+  static constexpr int TST = TK * 2 + 8;  // bytes per [d][key] row
+  static constexpr int ROW_BYTES = TK * KST;
+  static constexpr int T_BYTES = D * TST;
+  static constexpr int TILE_BYTES = 2 * ROW_BYTES + T_BYTES;  // K rows, V rows, K^T
+  static constexpr int OST = D * 2 + 16;
+};
+
+template <int D, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_kernel(BwdParams p) {
+  constexpr int NT = NW * 64;
+  constexpr int BM = NW * 32;
+  constexpr int CH = D / 8;
+  constexpr int UNITS = 16 * CH;
+  constexpr int PER = (UNITS + NT - 1) / NT;
+  constexpr int KK = D / 16;
+  constexpr int DB = D / 32;
+  using SM = DqSmem<D>;
+  static_assert(BM * SM::OST <= SM::TILE_BYTES, "dQ staging must fit the tile buffers");
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* Ks = smem;
+  unsigned char* Vs = smem + SM::ROW_BYTES;
+  unsigned char* Kt = smem + 2 * SM::ROW_BYTES;
+  u32x2* tdesc = (u32x2*)(smem + SM::TILE_BYTES);
+  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
+
+  const int I = blockIdx.x % p.Mq;
+  const int bh = blockIdx.x / p.Mq;
+  const int h = bh % p.Hq, b = bh / p.Hq;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal;
+  const float scale_log2 = p.scale_log2;
+
+  int jmax = p.Nk;
+  if (causal) {
+    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << bn_log2) - 1) >> bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  const int T = build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, bn_log2, L, causal != 0,
+                                       (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff);
+
+  // Q and dO fragments of this wave's 32 rows (B operands), per-row delta and lse
+  const int q_idx = I * BM + wave * 32 + l32;
+  const int qr = q_idx < L ? q_idx : L - 1;
+  bf16x8 qf[KK], dof[KK];
+  {
+    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+    const bf16_t* dp_ = p.dout + b * p.do_sb + h * p.do_sh + (int64_t)qr * p.do_sl + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qf[kk] = *(const bf16x8*)(qp + kk * 16);
+      dof[kk] = *(const bf16x8*)(dp_ + kk * 16);
+    }
+  }
+  const float delta = q_idx < L ? p.delta[(int64_t)bh * L + q_idx] : 0.f;
+  const float lse2 = q_idx < L ? p.lse2[(int64_t)bh * L + q_idx] : INFINITY;
+
+  const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
+  const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
+  const int64_t npad = p.npad;
+  const uint32_t k_strb = (uint32_t)p.k_sl * 2u, v_strb = (uint32_t)p.v_sl * 2u;
+  const bf16_t *kpool = p.kp, *vpool = p.vp;
+
+  u32x4 kreg[PER][4], vreg[PER][4];
+  auto load_tile = [&](int t) __attribute__((always_inline)) {
+    const TileRef r = tile_ref(tdesc, ids, t, bn_log2);
+    const int64_t prow = pool_row_offset(r.lv, BHkv, bhk, npad) * D;
+    const char* kbase = r.lv == 0 ? kb0 : (const char*)(kpool + prow);
+    const char* vbase = r.lv == 0 ? vb0 : (const char*)(vpool + prow);
+    const uint32_t ks = r.lv == 0 ? k_strb : (uint32_t)(D * 2);
+    const uint32_t vs = r.lv == 0 ? v_strb : (uint32_t)(D * 2);
+    const int lim = r.lv == 0 ? L : 0x7fffffff;
+#pragma unroll
+    for (int u_ = 0; u_ < PER; ++u_) {
+      const int u = tid + u_ * NT;
+      if (UNITS % NT != 0 && u >= UNITS) break;
+      const int r0 = (u & 15) * 4, ch = u >> 4;  // neighbouring lanes walk along the key quads of one chunk
+      const int src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, L);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int src = src0 + i;
+        src = (src0 >= 0 && src < lim) ? src : 0;  // empty slots: finite data, masked below
+        kreg[u_][i] = *(const u32x4*)(kbase + ((uint32_t)src * ks + (uint32_t)(ch * 16)));
+        vreg[u_][i] = *(const u32x4*)(vbase + ((uint32_t)src * vs + (uint32_t)(ch * 16)));
+      }
+    }
+  };
+  auto store_tile = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int u_ = 0; u_ < PER; ++u_) {
+      const int u = tid + u_ * NT;
+      if (UNITS % NT != 0 && u >= UNITS) break;
+      const int r0 = (u & 15) * 4, ch = u >> 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        *(u32x4*)(Ks + (r0 + i) * SM::KST + ch * 16) = kreg[u_][i];
+        *(u32x4*)(Vs + (r0 + i) * SM::KST + ch * 16) = vreg[u_][i];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {  // K^T: 4 keys x 8 channels -> 8 channels x 4 keys
+        u32x2 e0, e1;
+        e0[0] = __builtin_amdgcn_perm(kreg[u_][1][j], kreg[u_][0][j], 0x05040100u);
+        e0[1] = __builtin_amdgcn_perm(kreg[u_][3][j], kreg[u_][2][j], 0x05040100u);
+        e1[0] = __builtin_amdgcn_perm(kreg[u_][1][j], kreg[u_][0][j], 0x07060302u);
+        e1[1] = __builtin_amdgcn_perm(kreg[u_][3][j], kreg[u_][2][j], 0x07060302u);
+        *(u32x2*)(Kt + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
+        *(u32x2*)(Kt + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
+      }
+    }
+  };
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+
+  if (T > 0) load_tile(0);
+  for (int t = 0; t < T; ++t) {
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    const TileRef r = tile_ref(tdesc, ids, t, bn_log2);
+    if (t + 1 < T) load_tile(t + 1);
+
+    f32x16 s[2], dp[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[c][i] = 0.f;
+        dp[c][i] = 0.f;
+      }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const bf16x8 ka = *(const bf16x8*)(Ks + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
+        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s[c], 0, 0, 0);
+        const bf16x8 va = *(const bf16x8*)(Vs + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
+        dp[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp[c], 0, 0, 0);
+      }
+    }
+    if (r.masked) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int r0 = c * 32 + g * 8 + hh * 4;
+          int src0 = -1;
+          if (r0 < r.nvalid) src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, L);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool in_tile = src0 >= 0 && (r0 + e) < r.nvalid;
+            const bool visible = !causal || ((((int64_t)(src0 + e) + 1) << r.lv) - 1 <= (int64_t)q_idx);
+            const float sv = s[c][g * 4 + e];
+            s[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
+          }
+        }
+    }
+    const float nb = (float)r.lv - lse2;
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = fast_exp2(__builtin_fmaf(s[c][i], scale_log2, nb));
+        const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], scale_log2, nb));
+        pk[c][i >> 1] = pack_bf16x2(p0 * (dp[c][i] - delta), p1 * (dp[c][i + 1] - delta));
+      }
+    // dQ^T += K^T dS^T
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
+        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
+        const int key0 = c * 32 + g * 16 + hh * 4;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const unsigned char* kr = Kt + (db * 32 + l32) * SM::TST + key0 * 2;
+          const u32x2 lo = *(const u32x2*)(kr);
+          const u32x2 hi = *(const u32x2*)(kr + 16);
+          u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+        }
+      }
+  }
+
+  __syncthreads();
+  unsigned char* Os = smem;
+  const float scale = p.scale;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * scale, acc[db][g * 4 + 1] * scale);
+      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * scale, acc[db][g * 4 + 3] * scale);
+      *(u32x2*)(Os + (wave * 32 + l32) * SM::OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
+    }
+  __syncthreads();
+  bf16_t* ob = p.dq + b * p.dq_sb + h * p.dq_sh;
+  for (int u = tid; u < BM * CH; u += NT) {
+    const int rr = u / CH, ch = u % CH;
+    const int row = I * BM + rr;
+    if (row < L) *(u32x4*)(ob + (int64_t)row * p.dq_sl + ch * 8) = *(const u32x4*)(Os + rr * SM::OST + ch * 16);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------
+// dK, dV: column walk
+// ------------------------------------------------------------------------------------------------------
+template <int D>
+struct KvSmem {
+  static constexpr int RST = D * 2 + 16;   // bytes per [q][d] row
+  static constexpr int TST = 64 * 2 + 8;   // bytes per [d][q] row (64 query rows per step)
+  static constexpr int ROW_BYTES = 64 * RST;
+  static constexpr int T_BYTES = D * TST;
+  static constexpr int STAGE_BYTES = 2 * ROW_BYTES + 2 * T_BYTES;  // Q rows, dO rows, Q^T, dO^T
+};
+
+// slot -> (level, 64-key part inside the block); slots of a block: max(1, (bn>>lv)/64) per level
+__device__ __forceinline__ void decode_slot(int slot, int bn_log2, int& lv, int& part) {
+  lv = 0;
+  for (;;) {
+    const int n = (bn_log2 - lv) > 6 ? 1 << (bn_log2 - lv - 6) : 1;
+    if (slot < n) break;
+    slot -= n;
+    ++lv;
+  }
+  part = slot;
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int slots_per_block) {
+  constexpr int NT = 256;
+  constexpr int CH = D / 8;
+  constexpr int UNITS = 16 * CH;
+  constexpr int PER = (UNITS + NT - 1) / NT;
+  constexpr int KK = D / 16;
+  constexpr int DB = D / 32;
+  using SM = KvSmem<D>;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* Qs = smem;
+  unsigned char* Os = smem + SM::ROW_BYTES;
+  unsigned char* Qt = smem + 2 * SM::ROW_BYTES;
+  unsigned char* Ot = smem + 2 * SM::ROW_BYTES + SM::T_BYTES;
+  float* s_lse = (float*)(smem + SM::STAGE_BYTES);  // [64]
+  float* s_del = s_lse + 64;                        // [64]
+  uint32_t* qlist = (uint32_t*)(s_del + 64);        // [n_rep * Mq]  (head in group << 16 | q-block)
+  __shared__ int s_nq;
+
+  const int slot = blockIdx.x % slots_per_block;
+  const int J = blockIdx.x / slots_per_block;
+  const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  const int n_rep = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int kh = wave & 1, qh = wave >> 1;
+  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal, bm = p.bm, Mq = p.Mq;
+
+  int lv, part;
+  decode_slot(slot, bn_log2, lv, part);
+  const int sbs = 1 << (bn_log2 - lv);            // pooled keys of this block at this level
+  const int nkeys = sbs < 64 ? sbs : 64;
+  const int64_t key_row0 = ((int64_t)J << (bn_log2 - lv)) + part * 64;  // first pooled row of this workgroup
+  const int64_t n_lv = p.npad >> lv;
+  int key_valid = nkeys;                          // level 0: rows past L do not exist
+  if (lv == 0) {
+    const int64_t rem = (int64_t)L - key_row0;
+    key_valid = rem < nkeys ? (rem > 0 ? (int)rem : 0) : nkeys;
+  }
+
+  // ---- list of (head in group, q-block) that retain block J at this level -------------------------
+  if (wave == 0) {
+    int n = 0;
+    const int total = n_rep * Mq;
+    for (int e0 = 0; e0 < total; e0 += 64) {
+      const int e = e0 + lane;
+      bool on = false;
+      if (e < total) {
+        const int hl = e / Mq, I = e % Mq;
+        const int h = hk * n_rep + hl;
+        int level = p.map ? load_map(p.map, (((int64_t)b * p.Hq + h) * Mq + I) * p.Nk + J, p.map_elem) : 1;
+        if (causal) {
+          const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
+          if (J >= ce) level = 0;
+        }
+        on = level == (1 << lv);
+      }
+      const uint64_t bal = __ballot(on);
+      if (on) qlist[n + __popcll(bal & ((1ull << lane) - 1ull))] = ((uint32_t)(e / Mq) << 16) | (uint32_t)(e % Mq);
+      n += __popcll(bal);
+    }
+    if (lane == 0) s_nq = n;
+  }
+  __syncthreads();
+  const int nq = s_nq;
+
+  // ---- this wave's 32 keys: K and V fragments (B operands) --------------------------------------------
+  const int key_local = kh * 32 + l32;
+  bf16x8 kf[KK], vf[KK];
+  {
+    int64_t row = key_row0 + (key_local < key_valid ? key_local : 0);
+    if (key_valid == 0) row = 0;
+    const bf16_t *kp_, *vp_;
+    if (lv == 0) {
+      kp_ = p.k + b * p.k_sb + hk * p.k_sh + row * p.k_sl;
+      vp_ = p.v + b * p.v_sb + hk * p.v_sh + row * p.v_sl;
+    } else {
+      const int64_t off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + row) * D;
+      kp_ = p.kp + off;
+      vp_ = p.vp + off;
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      kf[kk] = *(const bf16x8*)(kp_ + kk * 16 + hh * 8);
+      vf[kk] = *(const bf16x8*)(vp_ + kk * 16 + hh * 8);
+    }
+  }
+  const bool key_ok = key_local < key_valid;
+  const int64_t key_up = ((key_row0 + key_local + 1) << lv) - 1;  // last token the pooled key covers
+
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      dk[db][i] = 0.f;
+      dv[db][i] = 0.f;
+    }
+  const float scale_log2 = p.scale_log2;
+  const float bias = (float)lv;
+  const int steps_per_block = bm / 64;
+
+  if (key_valid > 0) {
+    for (int e = 0; e < nq; ++e) {
+      const uint32_t ent = qlist[e];
+      const int h = hk * n_rep + (int)(ent >> 16), I = (int)(ent & 0xffff);
+      const int64_t bh = (int64_t)b * p.Hq + h;
+      const bool diag = causal && ((((int64_t)J + 1) << bn_log2) - 1 > (int64_t)I * bm);
+      for (int st = 0; st < steps_per_block; ++st) {
+        const int q0 = I * bm + st * 64;
+        if (q0 >= L) break;
+        __syncthreads();  // previous step's reads of the staging buffers are done
+        // stage 64 rows of Q and dO in both layouts
+#pragma unroll
+        for (int u_ = 0; u_ < PER; ++u_) {
+          const int u = tid + u_ * NT;
+          if (UNITS % NT != 0 && u >= UNITS) break;
+          const int r0 = (u & 15) * 4, ch = u >> 4;
+          u32x4 qreg[4], oreg[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            int row = q0 + r0 + i;
+            row = row < L ? row : L - 1;  // rows past L: p is forced to 0 through lse = +inf
+            qreg[i] = *(const u32x4*)(p.q + b * p.q_sb + h * p.q_sh + (int64_t)row * p.q_sl + ch * 8);
+            oreg[i] = *(const u32x4*)(p.dout + b * p.do_sb + h * p.do_sh + (int64_t)row * p.do_sl + ch * 8);
+            *(u32x4*)(Qs + (r0 + i) * SM::RST + ch * 16) = qreg[i];
+            *(u32x4*)(Os + (r0 + i) * SM::RST + ch * 16) = oreg[i];
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x2 e0, e1;
+            e0[0] = __builtin_amdgcn_perm(qreg[1][j], qreg[0][j], 0x05040100u);
+            e0[1] = __builtin_amdgcn_perm(qreg[3][j], qreg[2][j], 0x05040100u);
+            e1[0] = __builtin_amdgcn_perm(qreg[1][j], qreg[0][j], 0x07060302u);
+            e1[1] = __builtin_amdgcn_perm(qreg[3][j], qreg[2][j], 0x07060302u);
+            *(u32x2*)(Qt + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
+            *(u32x2*)(Qt + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
+            e0[0] = __builtin_amdgcn_perm(oreg[1][j], oreg[0][j], 0x05040100u);
+            e0[1] = __builtin_amdgcn_perm(oreg[3][j], oreg[2][j], 0x05040100u);
+            e1[0] = __builtin_amdgcn_perm(oreg[1][j], oreg[0][j], 0x07060302u);
+            e1[1] = __builtin_amdgcn_perm(oreg[3][j], oreg[2][j], 0x07060302u);
+            *(u32x2*)(Ot + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
+            *(u32x2*)(Ot + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
+          }
+        }
+        if (tid < 64) {
+          const int row = q0 + tid;
+          s_lse[tid] = row < L ? p.lse2[bh * L + row] : INFINITY;
+          s_del[tid] = row < L ? p.delta[bh * L + row] : 0.f;
+        }
+        __syncthreads();
+
+        // S = Q K^T and dP = dO V^T for this wave's (32 q) x (32 keys): lane = key column, registers = q rows
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s[i] = 0.f;
+          dp[i] = 0.f;
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const bf16x8 qa = *(const bf16x8*)(Qs + (qh * 32 + l32) * SM::RST + hh * 16 + kk * 32);
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
+          const bf16x8 oa = *(const bf16x8*)(Os + (qh * 32 + l32) * SM::RST + hh * 16 + kk * 32);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[kk], dp, 0, 0, 0);
+        }
+        uint32_t pk[8], dsk[8];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int qq = qh * 32 + g * 8 + hh * 4;
+          const f32x4 l4 = *(const f32x4*)(s_lse + qq);
+          const f32x4 d4 = *(const f32x4*)(s_del + qq);
+          float pv[4], dsv[4];
+#pragma unroll
+          for (int e2 = 0; e2 < 4; ++e2) {
+            float pe = fast_exp2(__builtin_fmaf(s[g * 4 + e2], scale_log2, bias - l4[e2]));
+            bool ok = key_ok;
+            if (diag) ok = ok && (key_up <= (int64_t)(q0 + qq + e2));
+            pe = ok ? pe : 0.f;
+            pv[e2] = pe;
+            dsv[e2] = pe * (dp[g * 4 + e2] - d4[e2]);
+          }
+          pk[g * 2] = pack_bf16x2(pv[0], pv[1]);
+          pk[g * 2 + 1] = pack_bf16x2(pv[2], pv[3]);
+          dsk[g * 2] = pack_bf16x2(dsv[0], dsv[1]);
+          dsk[g * 2 + 1] = pack_bf16x2(dsv[2], dsv[3]);
+        }
+        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over this wave's 32 query rows, 16 at a time)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
+          u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
+          const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
+          const int qq0 = qh * 32 + g * 16 + hh * 4;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const unsigned char* orow = Ot + (db * 32 + l32) * SM::TST + qq0 * 2;
+            const u32x2 olo = *(const u32x2*)(orow), ohi = *(const u32x2*)(orow + 16);
+            u32x4 oa = {olo[0], olo[1], ohi[0], ohi[1]};
+            dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, oa), pfrag, dv[db], 0, 0, 0);
+            const unsigned char* qrow = Qt + (db * 32 + l32) * SM::TST + qq0 * 2;
+            const u32x2 qlo = *(const u32x2*)(qrow), qhi = *(const u32x2*)(qrow + 16);
+            u32x4 qa2 = {qlo[0], qlo[1], qhi[0], qhi[1]};
+            dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qa2), sfrag, dk[db], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- combine the two query halves and write this workgroup's rows of the level buffers ------------
+  __syncthreads();
+  float* red = (float*)smem;  // [2 key halves][2 tensors][DB*16][64 lanes]
+  if (qh == 1) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane] = dk[db][i];
+        red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane] = dv[db][i];
+      }
+  }
+  __syncthreads();
+  if (qh == 0 && key_local < nkeys) {
+    const int64_t lvl_off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + (lv == 0 ? (int64_t)p.B * p.Hkv * 0 : 0));
+    // level buffers: level 0 first ([BHkv, npad, D]), then levels 1..3 like the pooled K/V buffers
+    const int64_t base_rows = lv == 0 ? bhk * p.npad : (int64_t)p.B * p.Hkv * p.npad + lvl_off;
+    float* wk = p.wk + (base_rows + key_row0 + key_local) * D;
+    float* wv = p.wv + (base_rows + key_row0 + key_local) * D;
+    const float scale = p.scale;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 a, c2;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int i = g * 4 + e2;
+          a[e2] = (dk[db][i] + red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane]) * scale;
+          c2[e2] = dv[db][i] + red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane];
+        }
+        *(f32x4*)(wk + db * 32 + g * 8 + hh * 4) = a;
+        *(f32x4*)(wv + db * 32 + g * 8 + hh * 4) = c2;
+      }
+  }
+  (void)n_lv;
+}
+
+// ------------------------------------------------------------------------------------------------------
+// un-pool: levels -> dK, dV (bf16)
+// ------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void psa_bwd_unpool_kernel(BwdParams p, int D) {
+  const int which = blockIdx.z;  // 0: dK, 1: dV
+  const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  const int chunks = D >> 2;  // float4 chunks per row
+  const int64_t unit = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t n = unit / chunks;
+  const int c = (int)(unit % chunks);
+  if (n >= p.L) return;
+  const float* w = which == 0 ? p.wk : p.wv;
+  const int64_t BH = (int64_t)p.B * p.Hkv, npad = p.npad;
+  const float* w0 = w + (bhk * npad) * D;
+  const float* wl[3];
+#pragma unroll
+  for (int lv = 1; lv < 4; ++lv) wl[lv - 1] = w + (BH * npad + pool_row_offset(lv, BH, bhk, npad)) * D;
+  auto contrib = [&](int64_t row) {
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int lv = 1; lv < 4; ++lv) {
+      const f32x4 x = *(const f32x4*)(wl[lv - 1] + (row >> lv) * D + c * 4);
+      const float inv = 1.0f / (float)(1 << lv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] += x[e] * inv;
+    }
+    return a;
+  };
+  f32x4 g = *(const f32x4*)(w0 + n * D + c * 4);
+  {
+    const f32x4 a = contrib(n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) g[e] += a[e];
+  }
+  if (n == p.L - 1) {  // gradient of the replicate-pad rows lands on the last real token
+    for (int64_t r = p.L; r < npad; ++r) {
+      const f32x4 a = contrib(r);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] += a[e];
+    }
+  }
+  bf16_t* dst = which == 0 ? p.dk + b * p.dk_sb + hk * p.dk_sh + n * p.dk_sl : p.dv + b * p.dv_sb + hk * p.dv_sh + n * p.dv_sl;
+  u32x2 o;
+  o[0] = pack_bf16x2(g[0], g[1]);
+  o[1] = pack_bf16x2(g[2], g[3]);
+  *(u32x2*)(dst + c * 4) = o;
+}
+
+int slots_of(int block_n) {
+  int n = 0;
+  for (int lv = 0; lv < 4; ++lv) n += (block_n >> lv) > 64 ? (block_n >> lv) / 64 : 1;
+  return n;
+}
+
+}  // namespace
+
+extern "C" int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || L <= 0 || D <= 0 || block_n <= 0) return 0;
+  const int64_t npad = (int64_t)((L + block_n - 1) / block_n) * block_n;
+  const int64_t levels = (int64_t)B * Hkv * D * (npad + npad / 2 + npad / 4 + npad / 8);
+  return (2 * levels + 2 * (int64_t)B * Hq * L) * (int64_t)sizeof(float);
+}
+
+extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool, const void* map,
+                       int map_elem_bytes, psa_tensor4 out, psa_tensor4 dout, const float* lse, psa_tensor4 dq, psa_tensor4 dk,
+                       psa_tensor4 dv, void* workspace, int B, int Hq, int Hkv, int L, int D, int block_m, int block_n,
+                       float sm_scale, int causal, psa_stream_t stream) {
+  PSA_REQUIRE(q.ptr && k.ptr && v.ptr && out.ptr && dout.ptr && lse && dq.ptr && dk.ptr && dv.ptr && workspace, PSA_ERR_ARG,
+              "psa_bwd: null pointer");
+  PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_bwd: pooled K/V required with a level map");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_bwd: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0, PSA_ERR_ARG, "psa_bwd: B, H, L must be positive");
+  PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_bwd: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
+  PSA_REQUIRE(sm_scale > 0.f, PSA_ERR_ARG, "psa_bwd: sm_scale must be positive");
+  PSA_REQUIRE(D == 64 || D == 128, PSA_ERR_UNSUPPORTED, "psa_bwd: head dim %d not in {64, 128}", D);
+  PSA_REQUIRE(block_m == 64 || block_m == 128, PSA_ERR_UNSUPPORTED, "psa_bwd: block_m=%d not in {64, 128}", block_m);
+  PSA_REQUIRE(block_n == 32 || block_n == 64 || block_n == 128, PSA_ERR_UNSUPPORTED, "psa_bwd: block_n=%d not in {32, 64, 128}", block_n);
+  const psa_tensor4* ts[8] = {&q, &k, &v, &out, &dout, &dq, &dk, &dv};
+  for (int i = 0; i < 8; ++i)
+    PSA_REQUIRE(((uintptr_t)ts[i]->ptr % 16 == 0) && ts[i]->stride_b % 8 == 0 && ts[i]->stride_h % 8 == 0 && ts[i]->stride_l % 8 == 0,
+                PSA_ERR_UNSUPPORTED, "psa_bwd: tensors must be 16-byte aligned with strides that are multiples of 8 elements");
+  PSA_REQUIRE((int64_t)L * k.stride_l * 2 < (1ll << 32) && (int64_t)L * v.stride_l * 2 < (1ll << 32), PSA_ERR_UNSUPPORTED,
+              "psa_bwd: one (batch, head) slice of K/V must span less than 4 GiB");
+  const int Mq = (L + block_m - 1) / block_m, Nk = (L + block_n - 1) / block_n;
+  PSA_REQUIRE(Nk <= 65535 && Mq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: more than 65535 blocks");
+  PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: B*Hq too large");
+  BwdParams p;
+  p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr; p.v = (const bf16_t*)v.ptr;
+  p.o = (const bf16_t*)out.ptr; p.dout = (const bf16_t*)dout.ptr;
+  p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sl = q.stride_l;
+  p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sl = k.stride_l;
+  p.v_sb = v.stride_b; p.v_sh = v.stride_h; p.v_sl = v.stride_l;
+  p.o_sb = out.stride_b; p.o_sh = out.stride_h; p.o_sl = out.stride_l;
+  p.do_sb = dout.stride_b; p.do_sh = dout.stride_h; p.do_sl = dout.stride_l;
+  p.dq = (bf16_t*)dq.ptr; p.dk = (bf16_t*)dk.ptr; p.dv = (bf16_t*)dv.ptr;
+  p.dq_sb = dq.stride_b; p.dq_sh = dq.stride_h; p.dq_sl = dq.stride_l;
+  p.dk_sb = dk.stride_b; p.dk_sh = dk.stride_h; p.dk_sl = dk.stride_l;
+  p.dv_sb = dv.stride_b; p.dv_sh = dv.stride_h; p.dv_sl = dv.stride_l;
+  p.kp = (const bf16_t*)k_pool; p.vp = (const bf16_t*)v_pool;
+  p.map = map; p.map_elem = map_elem_bytes; p.lse = lse;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.L = L; p.Mq = Mq; p.Nk = Nk;
+  p.bn_log2 = psa_ilog2(block_n); p.bm = block_m;
+  p.npad = (int64_t)Nk * block_n;
+  p.scale = sm_scale;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  p.causal = causal ? 1 : 0;
+  p.max_tiles = psa_tiles::max_tiles(Nk, block_n);
+  const int64_t levels = (int64_t)B * Hkv * D * (p.npad + p.npad / 2 + p.npad / 4 + p.npad / 8);
+  p.wk = (float*)workspace;
+  p.wv = p.wk + levels;
+  p.delta = p.wv + levels;
+  p.lse2 = p.delta + (int64_t)B * Hq * L;
+  hipStream_t st = (hipStream_t)stream;
+
+  // 1. delta, lse2
+  {
+    const int rows_per_wg = 256 / (D / 8);
+    dim3 grid((unsigned)((L + rows_per_wg - 1) / rows_per_wg), (unsigned)(B * Hq));
+    if (D == 128) hipLaunchKernelGGL(psa_bwd_delta_kernel<128>, grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(psa_bwd_delta_kernel<64>, grid, dim3(256), 0, st, p);
+    const int rc = psa_check_launch("psa_bwd (delta)");
+    if (rc != PSA_OK) return rc;
+  }
+  // 2. dQ
+  {
+    const int64_t total = (int64_t)B * Hq * Mq;
+    PSA_REQUIRE(total < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    auto launch = [&](auto kern, size_t tile_bytes, int nw) -> int {
+      const size_t shmem = tile_bytes + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
+      if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
+      if (shmem > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+        return PSA_ERR_LAUNCH;
+      hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(nw * 64), shmem, st, p);
+      return PSA_OK;
+    };
+    int rc;
+    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq_kernel<128, 4>, DqSmem<128>::TILE_BYTES, 4);
+    else if (D == 128) rc = launch(psa_bwd_dq_kernel<128, 2>, DqSmem<128>::TILE_BYTES, 2);
+    else if (block_m == 128) rc = launch(psa_bwd_dq_kernel<64, 4>, DqSmem<64>::TILE_BYTES, 4);
+    else rc = launch(psa_bwd_dq_kernel<64, 2>, DqSmem<64>::TILE_BYTES, 2);
+    PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: sequence too long for the on-chip schedule (LDS)");
+    rc = psa_check_launch("psa_bwd (dQ)");
+    if (rc != PSA_OK) return rc;
+  }
+  // 3. dK, dV per level
+  {
+    const int spb = slots_of(block_n);
+    const int n_rep = Hq / Hkv;
+    dim3 grid((unsigned)(Nk * spb), (unsigned)(B * Hkv));
+    auto launch = [&](auto kern, size_t stage_bytes) -> int {
+      size_t shmem = stage_bytes + 128 * sizeof(float) + (size_t)n_rep * Mq * 4;
+      const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
+      if (shmem < red) shmem = red;
+      if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
+      if (shmem > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+        return PSA_ERR_LAUNCH;
+      hipLaunchKernelGGL(kern, grid, dim3(256), shmem, st, p, spb);
+      return PSA_OK;
+    };
+    int rc = D == 128 ? launch(psa_bwd_dkdv_kernel<128>, KvSmem<128>::STAGE_BYTES) : launch(psa_bwd_dkdv_kernel<64>, KvSmem<64>::STAGE_BYTES);
+    PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
+    rc = psa_check_launch("psa_bwd (dK/dV)");
+    if (rc != PSA_OK) return rc;
+  }
+  // 4. un-pool
+  {
+    const int64_t units = (int64_t)L * (D / 4);
+    dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * Hkv), 2);
+    hipLaunchKernelGGL(psa_bwd_unpool_kernel, grid, dim3(256), 0, st, p, D);
+  }
+  return psa_check_launch("psa_bwd (un-pool)");
+}

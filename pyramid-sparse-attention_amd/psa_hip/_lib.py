@@ -49,6 +49,12 @@ SIGNATURES = {
         [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,
          c_int, c_int, c_int, c_float, c_int, c_void_p],
     ),
+    "psa_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "psa_bwd": (
+        c_int,
+        [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, Tensor4, c_void_p, Tensor4, Tensor4, Tensor4,
+         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    ),
 }
 
 

@@ -252,3 +252,51 @@ def sparse_attention_fwd(
     if return_lse:
         return res, lse, (kp, vp)
     return res
+
+
+# ----------------------------------------------------------------------------- attention backward
+def sparse_attention_bwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    level_map_: Optional[torch.Tensor],
+    out: torch.Tensor,
+    dout: torch.Tensor,
+    lse: torch.Tensor,
+    block_m: int,
+    block_n: int,
+    sm_scale: Optional[float] = None,
+    causal: bool = False,
+    pools: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+):
+    """dq, dk, dv of sparse_attention_fwd (dtype of q / k / v); lse is the fp32 [B,Hq,L] tensor the forward
+    returned.  The level map carries no gradient."""
+    _require_gpu(q, k, v, level_map_, out, dout, lse)
+    qb, kb, vb, ob, dob = (_bf16_view(t) for t in (q, k, v, out, dout))
+    B, Hq, L, D = qb.shape
+    Hkv = kb.shape[1]
+    sm_scale = D ** -0.5 if sm_scale is None else float(sm_scale)
+    Mq, Nk = -(-L // block_m), -(-L // block_n)
+    kp = vp = None
+    if level_map_ is not None:
+        if level_map_.dtype not in (torch.int8, torch.int32):
+            level_map_ = level_map_.to(torch.int32)
+        level_map_ = level_map_.contiguous()
+        if tuple(level_map_.shape) != (B, Hq, Mq, Nk):
+            raise ValueError("level map must be [B, Hq, %d, %d], got %s" % (Mq, Nk, tuple(level_map_.shape)))
+        kp, vp = pools if pools is not None and pools[0] is not None else pool_kv(kb, vb, block_n)
+    lse = lse.to(torch.float32).contiguous()
+    if tuple(lse.shape) != (B, Hq, L):
+        raise ValueError("lse must be [B, Hq, L]")
+    dq = torch.empty(B, Hq, L, D, dtype=torch.bfloat16, device=q.device)
+    dk = torch.empty(B, Hkv, L, D, dtype=torch.bfloat16, device=q.device)
+    dv = torch.empty(B, Hkv, L, D, dtype=torch.bfloat16, device=q.device)
+    ws = torch.empty(lib.psa_bwd_workspace_bytes(B, Hq, Hkv, L, D, block_n), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        check(
+            lib.psa_bwd(_t4(qb), _t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_),
+                        1 if level_map_ is None else level_map_.element_size(), _t4(ob), _t4(dob), _ptr(lse), _t4(dq), _t4(dk), _t4(dv),
+                        _ptr(ws), B, Hq, Hkv, L, D, block_m, block_n, sm_scale, int(causal), _stream(q)),
+            "psa_bwd",
+        )
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
