@@ -103,6 +103,14 @@ int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_
 int psa_map_from_list(const int32_t* list, void* map_out, int map_elem_bytes, int64_t rows,
                       int width, int Nk, psa_stream_t stream);
 
+/* Key-similarity cap: cap_out [B, H, Nk] int32 in {1, 2, 4, 8}.  For a kv-block, sim_l = mean cosine
+ * similarity of the token pairs (g*l, g*l + l-1); the cap is the largest l in {2, 4, 8} with
+ * sim_l > thr_l (strictly), else 1.  cos = a.b / (sqrt(|a|^2 + 1e-12) sqrt(|b|^2 + 1e-12) + 1e-6), fp32;
+ * tokens past L replicate token L-1.
+ * Replaces calc_k_similarity_triton: reference src/psa_triton/kernels/calc_ksim_kernel.py:6-157,160-225. */
+int psa_ksim(psa_tensor4 k, int32_t* cap_out, int B, int H, int L, int D, int block_n,
+             float thr2, float thr4, float thr8, psa_stream_t stream);
+
 /* out[i] = min(map[i], cap[col]) with cap [B*Hkv... given per (b, h, kv-block)] broadcast over q-blocks:
  * the "sim mask" clamp.  reference src/psa_triton/attention.py:296-299. */
 int psa_map_min_cap(void* map, int map_elem_bytes, const int32_t* cap, int64_t bh, int Mq, int Nk,

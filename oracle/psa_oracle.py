@@ -634,20 +634,35 @@ def estimate_xattn(q, k, block_size=128, stride=8, causal=True, chunk_size=4096,
 # --------------------------------------------------------------------------------------
 # K-similarity "sim mask"   reference: src/psa_triton/attention.py:140-164
 # --------------------------------------------------------------------------------------
-def k_similarity(k: torch.Tensor, block_n: int, thr2: float, thr4: float, thr8: float) -> torch.Tensor:
-    """Per kv-block cap on the pooling level: mean cosine similarity of token pairs at
-    distance 1 (even/odd), 3 (0::4 vs 3::4), 7 (0::8 vs 7::8); level = max over the
-    thresholds passed (strict >), at least 1.  k must already be padded to block_n."""
-    B, H, L, D = k.shape
+def k_similarity_scores(k: torch.Tensor, block_n: int):
+    """(sim2, sim4, sim8) [B,H,Nk] fp32: mean over the block of the cosine similarity of token pairs
+    (2g, 2g+1), (4g, 4g+3), (8g, 8g+7), with the GPU kernel's formula
+    cos = a.b / (sqrt(|a|^2 + 1e-12) * sqrt(|b|^2 + 1e-12) + 1e-6); tokens past L replicate the last.
+    reference: src/psa_triton/kernels/calc_ksim_kernel.py:66-137 (torch fallback: src/psa_triton/attention.py:140-164,
+    identical up to the epsilons)."""
+    kp = pad_replicate(k, block_n).float()
+    B, H, L, D = kp.shape
     nb = L // block_n
-    kc = k[:, :, : nb * block_n].float().reshape(B, H, nb, block_n, D)
-    s2 = F.cosine_similarity(kc[..., 0::2, :], kc[..., 1::2, :], dim=-1).mean(-1)
-    s4 = F.cosine_similarity(kc[..., 0::4, :], kc[..., 3::4, :], dim=-1).mean(-1)
-    s8 = F.cosine_similarity(kc[..., 0::8, :], kc[..., 7::8, :], dim=-1).mean(-1)
-    m2 = 2 * (s2 > thr2)
-    m4 = 4 * (s4 > thr4)
-    m8 = 8 * (s8 > thr8)
-    return torch.maximum(torch.ones_like(m2), torch.maximum(m2, torch.maximum(m4, m8))).to(torch.int32)
+    kc = kp.reshape(B, H, nb, block_n, D)
+    nrm = torch.sqrt((kc * kc).sum(-1) + 1e-12)
+
+    def sim(step):
+        a, b_ = kc[..., 0::step, :], kc[..., step - 1::step, :]
+        na, nb_ = nrm[..., 0::step], nrm[..., step - 1::step]
+        return ((a * b_).sum(-1) / (na * nb_ + 1e-6)).mean(-1)
+
+    return sim(2), sim(4), sim(8)
+
+
+def k_similarity(k: torch.Tensor, block_n: int, thr2: float, thr4: float, thr8: float) -> torch.Tensor:
+    """Per kv-block cap on the pooling level: the largest l in {2,4,8} whose similarity passes its
+    threshold (strict >), at least 1.  reference: src/psa_triton/kernels/calc_ksim_kernel.py:139-144."""
+    s2, s4, s8 = k_similarity_scores(k, block_n)
+    out = torch.ones_like(s2, dtype=torch.int32)
+    out = torch.where(s2 > thr2, torch.full_like(out, 2), out)
+    out = torch.where(s4 > thr4, torch.full_like(out, 4), out)
+    out = torch.where(s8 > thr8, torch.full_like(out, 8), out)
+    return out
 
 
 # --------------------------------------------------------------------------------------

@@ -42,6 +42,7 @@ SIGNATURES = {
          c_int, c_double, c_void_p],
     ),
     "psa_map_from_list": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_void_p]),
+    "psa_ksim": (c_int, [Tensor4, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p]),
     "psa_map_min_cap": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "psa_density": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "psa_fwd": (

@@ -175,6 +175,18 @@ def map_from_list(list_mask: torch.Tensor, Nk: int, map_dtype: torch.dtype = tor
     return out
 
 
+def k_similarity(k: torch.Tensor, block_n: int, thr2: float, thr4: float, thr8: float) -> torch.Tensor:
+    """Per kv-block cap on the pooling level, int32 [B,H,Nk] in {1,2,4,8}."""
+    _require_gpu(k)
+    kb = _bf16_view(k)
+    B, H, L, D = kb.shape
+    Nk = -(-L // block_n)
+    out = torch.empty(B, H, Nk, dtype=torch.int32, device=k.device)
+    with torch.cuda.device(k.device):
+        check(lib.psa_ksim(_t4(kb), _ptr(out), B, H, L, D, block_n, float(thr2), float(thr4), float(thr8), _stream(k)), "psa_ksim")
+    return out
+
+
 def map_min_cap(level_map_: torch.Tensor, cap: torch.Tensor) -> torch.Tensor:
     """In place: map[b,h,i,j] = min(map[b,h,i,j], cap[b,h,j])."""
     _require_gpu(level_map_, cap)
