@@ -97,6 +97,34 @@ int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_
                   const double* item_hi, int align_div, int text_blocks, double min_full_attn_ratio,
                   psa_stream_t stream);
 
+/* Level map of the causal Qwen2.5-VL example: scores [bh, S, S] fp32 -> map [bh, S, S].  Items (level, lo, hi) in
+ * dict order (host arrays).  PSA_MODE_TOPK: sorted positions [floor(len*lo), floor(len*hi)) get the level, len = row+1
+ * if causal else S; PSA_MODE_THRESHOLDBOUND ("energybound"): positions whose cumulative ratio r satisfies
+ * max(lo, previous hi) < r <= hi.  Then: the last special_blocks rows and columns := 1, the strict upper triangle := 0
+ * (causal), the diagonal := 1, column 0 := 1.  r = prefix sum / max(last prefix sum, 1e-10) with the prefix sums
+ * accumulated sequentially in fp64 over the sorted row (the reference divides by torch's sum of the unsorted row).
+ * Replaces the Qwen transfer_attn_to_mask:
+ *   reference qwen2.5-vl-example/src/attention/PSA_casual/PyramidAdaptiveBlockSparseAttn.py:84-168. */
+int psa_level_map_qwen(const float* scores, void* map_out, int map_elem_bytes, int64_t bh, int S, int mode,
+                       int n_items, const int32_t* item_level, const double* item_lo, const double* item_hi,
+                       int special_blocks, int causal, psa_stream_t stream);
+
+/* Bytes of scratch psa_estimate_xattn needs. */
+int64_t psa_estimate_xattn_workspace_bytes(int B, int Hq, int Lq, int Lk, int block_size, int stride,
+                                           int chunk_size);
+
+/* Antidiagonal ("xattn") block-importance estimate of the causal Qwen2.5-VL path:
+ * A[m,n] = sum_{i<stride} q[m*stride + stride-1-i] . k[n*stride + i], logits A / (sqrt(D) * stride), causal n <= m
+ * (key-aligned), row softmax over all strided keys, probabilities summed inside (block_size/stride)^2 cells.
+ * q, k are zero-padded to a multiple of chunk_size tokens; est [B, Hq, ceil(Lq/block), ceil(Lk/block)] fp32.
+ * K has Hkv heads (query head h uses kv head h / (Hq/Hkv)); the logits never reach HBM.
+ * Replaces estimate_block_importance's Triton path:
+ *   reference qwen2.5-vl-example/src/attention/PSA_casual/utils/block_importance.py:282-562,
+ *   qwen2.5-vl-example/src/attention/PSA_casual/kernels/block_importance_kernels.py:6-192,255-323. */
+int psa_estimate_xattn(psa_tensor4 q, psa_tensor4 k, float* est, void* workspace, int B, int Hq, int Hkv,
+                       int Lq, int Lk, int D, int block_size, int stride, int chunk_size, int causal,
+                       psa_stream_t stream);
+
 /* Index list ("new mask type", [rows, width] int32) -> dense level map [rows, Nk], read the way the
  * reference's list-walking kernel reads it: segment level starts at 1, doubles at every -1, stops
  * after 8.  reference src/psa_triton/kernels/psa_kernel.py:207-217. */

@@ -386,13 +386,16 @@ def level_map_qwen(
         valid = (np.arange(S, dtype=np.float32) + 1.0) if causal else np.full(S, float(S), np.float32)
         valid = valid.reshape(1, 1, S, 1)
         for lv, (lo, hi) in mask_ratios.items():
-            s = np.floor(valid * np.float32(lo)).astype(np.int64)
-            e = np.floor(valid * np.float32(hi)).astype(np.int64)
+            s = np.minimum(np.floor(valid * np.float32(lo)).astype(np.int64), S)
+            e = np.minimum(np.floor(valid * np.float32(hi)).astype(np.int64), S)
             sel = (pos >= s) & (pos < e)
             sorted_lv = np.where(sel, np.int32(lv), sorted_lv)
     elif mode == "energybound":
-        total = np.maximum(scores.sum(-1, keepdims=True, dtype=np.float32), np.float32(1e-10))
+        # contract of this build: the row total is the last prefix sum (sequential fp64 accumulation over the sorted
+        # row, rounded to fp32); the reference divides by torch's fp32 sum of the unsorted row (:134), whose
+        # summation order is an implementation detail of the library
         c = np.cumsum(w.astype(np.float64), -1).astype(np.float32)
+        total = np.maximum(c[..., -1:], np.float32(1e-10))
         r = c / total
         prev_hi = 0.0
         for lv, (lo, hi) in mask_ratios.items():

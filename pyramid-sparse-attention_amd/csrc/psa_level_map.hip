@@ -219,6 +219,117 @@ extern "C" int psa_level_map(const float* scores, void* map_out, int map_elem_by
 }
 
 // ---------------------------------------------------------------------------------------
+// level map of the causal Qwen2.5-VL example: square map, per-row ratio windows, fix-ups
+// ---------------------------------------------------------------------------------------
+struct QwenMapParams {
+  const float* scores;
+  void* map_out;
+  int map_elem;
+  int S;       // blocks per side
+  int mode;    // PSA_MODE_TOPK: rank windows on the causal row length; PSA_MODE_THRESHOLDBOUND: cumulative-mass windows
+  int n_items;
+  int level[PSA_MAX_LEVEL_ITEMS];
+  float lo[PSA_MAX_LEVEL_ITEMS];  // energy mode: max(lo, previous hi); rank mode: lo
+  float hi[PSA_MAX_LEVEL_ITEMS];
+  int special;  // trailing blocks (rows and columns) forced to level 1
+  int causal;
+};
+
+__global__ __launch_bounds__(256) void psa_level_map_qwen_kernel(QwenMapParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int N = p.S;
+  uint64_t* key = (uint64_t*)smem;
+  float* sw = (float*)(key + N);
+  int* sidx = (int*)(sw + N);
+  float* c32 = (float*)(sidx + N);
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t row = blockIdx.x;
+  const int i_row = (int)(row % N);
+  const float* src = p.scores + row * N;
+  for (int j = tid; j < N; j += nt) key[j] = ((uint64_t)desc_key(src[j]) << 32) | (uint32_t)j;
+  __syncthreads();
+  for (int j = tid; j < N; j += nt) {
+    const uint64_t kj = key[j];
+    int rank = 0;
+    for (int i = 0; i < N; ++i) rank += key[i] < kj ? 1 : 0;
+    sw[rank] = src[j];
+    sidx[rank] = j;
+  }
+  __syncthreads();
+  if (p.mode == PSA_MODE_THRESHOLDBOUND) {
+    if (tid == 0) {
+      double acc = 0.0;
+      for (int i = 0; i < N; ++i) {
+        acc += (double)sw[i];
+        c32[i] = (float)acc;
+      }
+    }
+    __syncthreads();
+  }
+  const float total = p.mode == PSA_MODE_THRESHOLDBOUND ? fmaxf(c32[N - 1], 1e-10f) : 1.f;
+  const float valid_len = p.causal ? (float)(i_row + 1) : (float)N;
+  for (int pos = tid; pos < N; pos += nt) {
+    int lv = 0;
+    if (p.mode == PSA_MODE_THRESHOLDBOUND) {
+      const float r = c32[pos] / total;
+      for (int t = 0; t < p.n_items; ++t)
+        if (r > p.lo[t] && r <= p.hi[t]) lv = p.level[t];
+    } else {
+      for (int t = 0; t < p.n_items; ++t) {
+        int s0 = (int)(valid_len * p.lo[t]), e0 = (int)(valid_len * p.hi[t]);
+        s0 = s0 < N ? s0 : N;
+        e0 = e0 < N ? e0 : N;
+        if (pos >= s0 && pos < e0) lv = p.level[t];
+      }
+    }
+    const int col = sidx[pos];
+    if (col >= N - p.special || i_row >= N - p.special) lv = 1;
+    if (p.causal && col > i_row) lv = 0;
+    if (col == i_row || col == 0) lv = 1;
+    store_map(p.map_out, row * N + col, p.map_elem, lv);
+  }
+}
+
+extern "C" int psa_level_map_qwen(const float* scores, void* map_out, int map_elem_bytes, int64_t bh, int S, int mode,
+                                  int n_items, const int32_t* item_level, const double* item_lo, const double* item_hi,
+                                  int special_blocks, int causal, psa_stream_t stream) {
+  PSA_REQUIRE(scores && map_out && item_level && item_lo && item_hi, PSA_ERR_ARG, "psa_level_map_qwen: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_level_map_qwen: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(mode == PSA_MODE_TOPK || mode == PSA_MODE_THRESHOLDBOUND, PSA_ERR_ARG, "mode must be 'topk' or 'energybound'");
+  PSA_REQUIRE(n_items >= 1 && n_items <= PSA_MAX_LEVEL_ITEMS, PSA_ERR_ARG, "mask_ratios must not be empty (1..%d items)", PSA_MAX_LEVEL_ITEMS);
+  PSA_REQUIRE(bh > 0 && S > 0 && S <= 6144 && bh * S < (1ll << 31), PSA_ERR_UNSUPPORTED, "psa_level_map_qwen: sizes out of range");
+  QwenMapParams p;
+  p.scores = scores; p.map_out = map_out; p.map_elem = map_elem_bytes; p.S = S; p.mode = mode; p.n_items = n_items;
+  p.special = special_blocks < 0 ? 0 : (special_blocks > S ? S : special_blocks);
+  p.causal = causal ? 1 : 0;
+  double prev_hi = 0.0;
+  for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t) {
+    p.level[t] = 0; p.lo[t] = 0.f; p.hi[t] = 0.f;
+  }
+  for (int t = 0; t < n_items; ++t) {
+    const int lv = item_level[t];
+    PSA_REQUIRE(lv == 0 || lv == 1 || lv == 2 || lv == 4 || lv == 8, PSA_ERR_ARG, "psa_level_map_qwen: level %d not in {0,1,2,4,8}", lv);
+    p.level[t] = lv;
+    if (mode == PSA_MODE_THRESHOLDBOUND) {
+      const double lower = item_lo[t] > prev_hi ? item_lo[t] : prev_hi;
+      prev_hi = item_hi[t];
+      p.lo[t] = (float)lower;
+    } else {
+      p.lo[t] = (float)item_lo[t];
+    }
+    p.hi[t] = (float)item_hi[t];
+  }
+  size_t shmem = (size_t)S * 20;
+  if (shmem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_qwen_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map_qwen: cannot reserve %zu bytes of LDS", shmem);
+  }
+  const int nt = S <= 64 ? 64 : (S <= 128 ? 128 : 256);
+  hipLaunchKernelGGL(psa_level_map_qwen_kernel, dim3((unsigned)(bh * S)), dim3(nt), shmem, (hipStream_t)stream, p);
+  return psa_check_launch("psa_level_map_qwen");
+}
+
+// ---------------------------------------------------------------------------------------
 // index list -> dense map
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void psa_map_from_list_kernel(const int32_t* list, void* map, int map_elem, int width, int Nk) {

@@ -41,6 +41,16 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int,
          c_int, c_double, c_void_p],
     ),
+    "psa_level_map_qwen": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), POINTER(c_double), c_int, c_int,
+         c_void_p],
+    ),
+    "psa_estimate_xattn_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "psa_estimate_xattn": (
+        c_int,
+        [Tensor4, Tensor4, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ),
     "psa_map_from_list": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_void_p]),
     "psa_ksim": (c_int, [Tensor4, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p]),
     "psa_map_min_cap": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),

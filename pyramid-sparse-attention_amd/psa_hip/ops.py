@@ -163,6 +163,47 @@ def level_map(
     return out
 
 
+def level_map_qwen(scores: torch.Tensor, mask_ratios, text_length: int, mode: str, *, block_size: int, causal: bool,
+                   map_dtype: torch.dtype = torch.int32) -> torch.Tensor:
+    """Square causal level map of the Qwen2.5-VL example: scores [B,H,S,S] -> map [B,H,S,S]."""
+    if not mask_ratios:
+        raise ValueError("mask_ratios must not be empty")
+    if mode not in {"topk", "energybound"}:
+        raise ValueError("mode must be 'topk' or 'energybound'")
+    _require_gpu(scores)
+    s = scores.to(torch.float32).contiguous()
+    B, H, S, S2 = s.shape
+    if S != S2:
+        raise ValueError("scores must be square [B, H, S, S]")
+    items = list(mask_ratios.items())
+    n = len(items)
+    lv = (ctypes.c_int32 * n)(*[int(i[0]) for i in items])
+    lo = (ctypes.c_double * n)(*[float(i[1][0]) for i in items])
+    hi = (ctypes.c_double * n)(*[float(i[1][1]) for i in items])
+    special = min(-(-text_length // block_size) if text_length > 0 else 0, S)
+    out = torch.empty(B, H, S, S, dtype=map_dtype, device=s.device)
+    m = _lib.PSA_MODE_TOPK if mode == "topk" else _lib.PSA_MODE_THRESHOLDBOUND
+    with torch.cuda.device(s.device):
+        check(lib.psa_level_map_qwen(_ptr(s), _ptr(out), out.element_size(), B * H, S, m, n, lv, lo, hi, special, int(causal), _stream(s)),
+              "psa_level_map_qwen")
+    return out
+
+
+def estimate_xattn(q: torch.Tensor, k: torch.Tensor, block_size: int = 128, stride: int = 8, causal: bool = True,
+                   chunk_size: int = 4096) -> torch.Tensor:
+    """Antidiagonal block-importance estimate, fp32 [B,Hq,ceil(Lq/block),ceil(Lk/block)]."""
+    _require_gpu(q, k)
+    qb, kb = _bf16_view(q), _bf16_view(k)
+    B, Hq, Lq, D = qb.shape
+    Hkv, Lk = kb.shape[1], kb.shape[2]
+    est = torch.empty(B, Hq, -(-Lq // block_size), -(-Lk // block_size), dtype=torch.float32, device=q.device)
+    ws = torch.empty(lib.psa_estimate_xattn_workspace_bytes(B, Hq, Lq, Lk, block_size, stride, chunk_size), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        check(lib.psa_estimate_xattn(_t4(qb), _t4(kb), _ptr(est), _ptr(ws), B, Hq, Hkv, Lq, Lk, D, block_size, stride, chunk_size,
+                                     int(causal), _stream(q)), "psa_estimate_xattn")
+    return est
+
+
 def map_from_list(list_mask: torch.Tensor, Nk: int, map_dtype: torch.dtype = torch.int8) -> torch.Tensor:
     """Index list [..., W] int32 -> dense level map [..., Nk]."""
     _require_gpu(list_mask)
