@@ -161,7 +161,14 @@ int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk,
 int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
             const void* map, int map_elem_bytes, psa_tensor4 out, float* lse,
             int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
-            int causal, psa_stream_t stream);
+            int causal, void* workspace, psa_stream_t stream);
+
+/* Bytes of the optional psa_fwd workspace.  With it, rows of the level map are issued longest first
+ * (per share of the chip), which shortens the tail of the launch when rows retain different numbers of
+ * blocks; results are identical with and without it.  workspace == NULL issues rows in natural order.
+ * The reference balances load through the Triton launch grid alone
+ * (src/psa_triton/kernels/psa_kernel.py:398-431). */
+int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m);
 
 /* Bytes of workspace psa_bwd needs (fp32 dK/dV per pyramid level, delta, lse in log2 units). */
 int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n);

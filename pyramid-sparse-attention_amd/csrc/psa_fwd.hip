@@ -20,9 +20,9 @@
 //  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m); the running maximum is
 //    only raised when it grows by more than 2^8 would overflow nothing (lazy rescaling), so most
 //    tiles skip the accumulator rescale.
-//  * Software pipeline, one barrier per tile: while the softmax of tile t runs on the VALU the
-//    MFMA pipe computes S^T of tile t+1; K tiles t+2 and V tiles t+1 are written to the other LDS
-//    buffers and the global loads of K tile t+3 / V tile t+2 are in flight.
+//  * One barrier per tile: while tile t is computed from one pair of LDS buffers, tile t+1 is written
+//    to the other pair and the global loads of tile t+2 are in flight; inside a tile the LDS operand
+//    reads run one MFMA step ahead.  Two workgroups per CU overlap one's softmax with the other's MFMAs.
 //
 // Roofline: MFMA-bound; 4*BM*64*D flops per tile.
 #include "psa_common.h"
@@ -46,6 +46,7 @@ struct FwdParams {
   int causal;
   int total_wg, wg_chunk;
   int max_tiles;
+  const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
 };
 
 template <int D>
@@ -122,8 +123,9 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   // XCD-aware decode: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous range of (b, h, q-block) so that one XCD's L2 sees few heads at a time.
   const int bid = blockIdx.x;
-  const int logical = (bid & 7) * p.wg_chunk + (bid >> 3);
-  if (logical >= p.total_wg) return;
+  int logical = (bid & 7) * p.wg_chunk + (bid >> 3);
+  if (p.order != nullptr) logical = p.order[logical];
+  if (logical < 0 || logical >= p.total_wg) return;
   const int I = logical % p.Mq;
   const int bh = logical / p.Mq;
   const int h = bh % p.Hq, b = bh / p.Hq;
@@ -296,22 +298,6 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
       }
     }
   };
-  auto qk_tile = [&](const unsigned char* Ks, f32x16 (&s)[2]) {
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
-    // the two 32-key chunks are independent accumulation chains: interleave them
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const bf16x8 a = *(const bf16x8*)(Ks + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
-        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s[c], 0, 0, 0);
-      }
-    }
-  };
-
   // ---- 4. main loop -------------------------------------------------------------------------
   f32x16 acc[DB];
 #pragma unroll
@@ -324,31 +310,48 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   if (T > 0) {
     __syncthreads();  // tile descriptors visible
     u32x4 kreg[PER][4], vreg[PER][4];
-    f32x16 s_a[2], s_b[2];
     const int Tm1 = T - 1;
     auto clampt = [&](int t) __attribute__((always_inline)) { return t < Tm1 ? t : Tm1; };
-    // prologue: K(0), V(0) -> LDS; S(0); K(1) -> LDS; {K(2), V(1)} in flight
+    // prologue: tile 0 -> LDS buffers 0, tile 1 in flight
     load_rows(0, kb0, P_k_sl, P_kp, kreg, false);
     load_rows(0, vb0, P_v_sl, P_vp, vreg, true);
     store_k(Kbuf(0), kreg);
     store_vt(Vbuf(0), vreg);
     load_rows(clampt(1), kb0, P_k_sl, P_kp, kreg, false);
-    __syncthreads();
-    qk_tile(Kbuf(0), s_a);
-    store_k(Kbuf(1), kreg);
-    load_rows(clampt(2), kb0, P_k_sl, P_kp, kreg, false);
     load_rows(clampt(1), vb0, P_v_sl, P_vp, vreg, true);
     __syncthreads();
 
-    auto step = [&](int t, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2]) {
-      // invariant: s_cur = raw S^T of tile t; Kbuf((t+1)&1) = K(t+1); Vbuf(t&1) = V(t);
-      //            kreg = K(t+2), vreg = V(t+1) (loads in flight)
+    for (int t = 0; t < T; ++t) {
+      // invariant: LDS buffers t&1 hold tile t; kreg/vreg hold tile t+1 (loads issued one step ago)
       const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
       const int lv = d & 3;
-      store_k(Kbuf(t), kreg);
+      store_k(Kbuf(t + 1), kreg);
       store_vt(Vbuf(t + 1), vreg);
-      load_rows(clampt(t + 3), kb0, P_k_sl, P_kp, kreg, false);
+      load_rows(clampt(t + 2), kb0, P_k_sl, P_kp, kreg, false);
       load_rows(clampt(t + 2), vb0, P_v_sl, P_vp, vreg, true);
+
+      // S^T = K Q^T: two independent 32-key accumulation chains; LDS operands are fetched one k-step ahead
+      const unsigned char* Ks = Kbuf(t) + l32 * SM::KST + hh * 16;
+      f32x16 s_cur[2];
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_cur[c][i] = 0.f;
+      {
+        bf16x8 a0 = *(const bf16x8*)(Ks), a1 = *(const bf16x8*)(Ks + 32 * SM::KST);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          bf16x8 n0 = a0, n1 = a1;
+          if (kk + 1 < KK) {
+            n0 = *(const bf16x8*)(Ks + (kk + 1) * 32);
+            n1 = *(const bf16x8*)(Ks + 32 * SM::KST + (kk + 1) * 32);
+          }
+          s_cur[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s_cur[0], 0, 0, 0);
+          s_cur[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s_cur[1], 0, 0, 0);
+          a0 = n0;
+          a1 = n1;
+        }
+      }
 
       if (d & 4) {  // partly empty tile and/or causal diagonal: mask individual keys
         const TileRef r = tile_ref(t);
@@ -371,15 +374,10 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
           }
       }
 
-      // next tile's scores on the MFMA pipe while this tile's softmax runs on the VALU
-      __builtin_amdgcn_s_setprio(1);
-      qk_tile(Kbuf(t + 1), s_nxt);
-      __builtin_amdgcn_s_setprio(0);
-
       // online softmax of tile t (per query column = per lane, both half-waves)
       float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
 #pragma unroll
-      for (int i = 1; i < 16; ++i) mx = max3f(mx, s_cur[0][i], s_cur[1][i]);
+      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s_cur[0][i], s_cur[1][i]));
       mx = fmaxf(mx, shfl_xor32(mx));
       const float bias = (float)lv;
       const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
@@ -412,33 +410,42 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
           for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
       }
 
-      // O^T += V^T P^T : per 16-key group g, A = V^T[32 d][16 keys], B = P^T[16 keys][32 q]
-      const unsigned char* Vt = Vbuf(t);
-      __builtin_amdgcn_s_setprio(1);
+      // O^T += V^T P^T : per 16-key group g, A = V^T[32 d][16 keys], B = P^T[16 keys][32 q];
+      // the V^T operands of the next group are fetched while the current group's MFMAs issue
+      const unsigned char* Vt = Vbuf(t) + l32 * SM::VST + hh * 8;
+      u32x2 vlo[DB], vhi[DB];
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
+      for (int db = 0; db < DB; ++db) {
+        vlo[db] = *(const u32x2*)(Vt + db * 32 * SM::VST);
+        vhi[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + 16);
+      }
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
-          const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
-          const int key0 = c * 32 + g * 16 + hh * 4;
+      for (int cg = 0; cg < 4; ++cg) {
+        const int c = cg >> 1, g = cg & 1;
+        u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
+        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
+        u32x2 nlo[DB], nhi[DB];
 #pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            const unsigned char* vr = Vt + (db * 32 + l32) * SM::VST + key0 * 2;
-            const u32x2 lo = *(const u32x2*)(vr);
-            const u32x2 hi = *(const u32x2*)(vr + 16);
-            u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
-            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+        for (int db = 0; db < DB; ++db) {
+          nlo[db] = vlo[db];
+          nhi[db] = vhi[db];
+          if (cg + 1 < 4) {
+            nlo[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + (cg + 1) * 32);
+            nhi[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + (cg + 1) * 32 + 16);
           }
         }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          u32x4 aw = {vlo[db][0], vlo[db][1], vhi[db][0], vhi[db][1]};
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          vlo[db] = nlo[db];
+          vhi[db] = nhi[db];
+        }
       }
-      __builtin_amdgcn_s_setprio(0);
       __syncthreads();
-    };
-    // two tiles per trip: the S^T buffers swap roles without being copied
-    for (int t = 0; t < T; t += 2) {
-      step(t, s_a, s_b);
-      if (t + 1 < T) step(t + 1, s_b, s_a);
     }
   }
 
@@ -470,6 +477,64 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   }
 }
 
+// ---- longest-rows-first ordering ---------------------------------------------------------------------
+// Rows of the level map differ in the number of tiles they retain.  Workgroup ids are dealt round-robin
+// to the 8 XCDs and each XCD runs its ids in order, so sorting every XCD's share by decreasing tile count
+// shortens the tail of the launch.  The order only changes WHEN a row is computed, never its result.
+constexpr int COST_BINS = 2048;
+
+__global__ __launch_bounds__(256) void psa_fwd_cost_kernel(const void* map, int map_elem, int total, int Mq, int Nk, int bn_log2,
+                                                         int bm, int causal, int32_t* cost) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= total) return;
+  const int I = row % Mq;
+  int jmax = Nk;
+  if (causal) {
+    const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  int cnt[4] = {0, 0, 0, 0};
+  for (int j0 = 0; j0 < jmax; j0 += 64) {
+    const int j = j0 + lane;
+    const int lvl = j < jmax ? load_map(map, (int64_t)row * Nk + j, map_elem) : 0;
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
+  }
+  if (lane == 0) {
+    int tiles = 0;
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) tiles += ((cnt[lv] << (bn_log2 - lv)) + 63) >> 6;
+    cost[row] = tiles < COST_BINS - 1 ? tiles : COST_BINS - 1;
+  }
+}
+
+// one workgroup per XCD share: counting sort by decreasing cost
+__global__ __launch_bounds__(256) void psa_fwd_sort_kernel(const int32_t* cost, int total, int chunk, int32_t* order) {
+  __shared__ int hist[COST_BINS];
+  const int x = blockIdx.x, tid = threadIdx.x;
+  const int r0 = x * chunk;
+  for (int i = tid; i < COST_BINS; i += 256) hist[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < chunk; i += 256)
+    if (r0 + i < total) atomicAdd(&hist[cost[r0 + i]], 1);
+  __syncthreads();
+  if (tid == 0) {  // start offset of every bin, highest cost first
+    int run = 0;
+    for (int b = COST_BINS - 1; b >= 0; --b) {
+      const int c = hist[b];
+      hist[b] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < chunk; i += 256) {
+    if (r0 + i < total) order[r0 + atomicAdd(&hist[cost[r0 + i]], 1)] = r0 + i;
+  }
+  // ids past the last row of the last share
+  const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;
+  for (int i = valid + tid; i < chunk; i += 256) order[r0 + i] = -1;
+}
+
 template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   using SM = Smem<D>;
@@ -485,9 +550,15 @@ int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
 
 }  // namespace
 
+extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
+  if (B <= 0 || Hq <= 0 || L <= 0 || block_m <= 0) return 0;
+  const int64_t total = (int64_t)B * Hq * ((L + block_m - 1) / block_m);
+  return 2 * 8 * ((total + 7) / 8) * (int64_t)sizeof(int32_t);
+}
+
 extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
                        const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
-                       int D, int block_m, int block_n, float sm_scale, int causal, psa_stream_t stream) {
+                       int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
   PSA_REQUIRE(q.ptr && k.ptr && v.ptr && out.ptr, PSA_ERR_ARG, "psa_fwd: null pointer");
   PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_fwd: pooled K/V required with a level map");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
@@ -524,6 +595,18 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.wg_chunk = (int)((total + 7) / 8);
   // worst case: every kv-block at level 1, plus one partly filled tile per pooled level
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
+  p.order = nullptr;
+  if (workspace != nullptr && map != nullptr && total > 8 * 32) {
+    PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
+    int32_t* order = (int32_t*)workspace;
+    int32_t* cost = order + (int64_t)p.wg_chunk * 8;
+    hipLaunchKernelGGL(psa_fwd_cost_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes,
+                       (int)total, Mq, Nk, p.bn_log2, block_m, p.causal, cost);
+    if (int e = psa_check_launch("psa_fwd (row cost)")) return e;
+    hipLaunchKernelGGL(psa_fwd_sort_kernel, dim3(8), dim3(256), 0, (hipStream_t)stream, cost, (int)total, p.wg_chunk, order);
+    if (int e = psa_check_launch("psa_fwd (row order)")) return e;
+    p.order = order;
+  }
   int rc;
   if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
   else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);

@@ -267,9 +267,11 @@ def sparse_attention_fwd(
     return_lse: bool = False,
     pools: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
     out: Optional[torch.Tensor] = None,
+    balance: bool = True,
 ):
     """Pyramid sparse attention forward.  level_map_ None = dense attention.  Returns out (dtype and
-    shape of q) or (out, lse fp32 [B,H,L], (k_pool, v_pool))."""
+    shape of q) or (out, lse fp32 [B,H,L], (k_pool, v_pool)).  balance=True issues the rows of the map
+    longest first (same results, shorter tail)."""
     _require_gpu(q, k, v, level_map_)
     in_dtype = q.dtype
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
@@ -294,11 +296,14 @@ def sparse_attention_fwd(
     else:
         o = out
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
+    ws = None
+    if level_map_ is not None and balance:
+        ws = torch.empty(lib.psa_fwd_workspace_bytes(B, Hq, L, block_m) // 4, dtype=torch.int32, device=q.device)
     with torch.cuda.device(q.device):
         check(
             lib.psa_fwd(_t4(qb), _t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_),
                         1 if level_map_ is None else level_map_.element_size(), _t4(o), _ptr(lse), B, Hq, Hkv, L, D,
-                        block_m, block_n, sm_scale, int(causal), _stream(q)),
+                        block_m, block_n, sm_scale, int(causal), _ptr(ws), _stream(q)),
             "psa_fwd",
         )
     res = o if in_dtype == torch.bfloat16 else o.to(in_dtype)

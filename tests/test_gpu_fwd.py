@@ -134,3 +134,32 @@ def test_fwd_errors():
         ops.sparse_attention_fwd(q, q, q, torch.ones(1, 1, 2, 1, dtype=torch.int8, device=dev()), 128, 128)  # map shape
     with pytest.raises(ValueError):
         ops.sparse_attention_fwd(q, q, q, None, 100, 128)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_longest_first_order_is_a_pure_reordering(causal):
+    """With the workspace the rows are issued longest first; every row must still be computed exactly
+    once and bit-identically (the unordered launch is the one checked against the oracle above)."""
+    from psa_hip import ops
+
+    B, H, L, D, bm, bn = 1, 5, 128 * 67 + 40, 128, 128, 128
+    Mq, Nk = -(-L // bm), -(-L // bn)
+    rng = np.random.default_rng(5)
+    lmap = random_map(B, H, Mq, Nk, 11)
+    # strongly uneven rows: some empty, some full
+    keep = rng.random((B, H, Mq, 1)) ** 2
+    lmap = np.where(rng.random(lmap.shape) < keep, lmap, 0).astype(lmap.dtype)
+    lmap[:, :, 3] = 0
+    lmap[:, :, 7] = 1
+    q, k, v = (rnd(B, H, L, D, seed=s).to(dev()) for s in (1, 2, 3))
+    m = torch.from_numpy(lmap).to(dev())
+    outs = []
+    for balance in (False, True):
+        o = torch.full((B, H, L, D), float("nan"), dtype=torch.bfloat16, device=dev())
+        res, lse, _ = ops.sparse_attention_fwd(q, k, v, m, bm, bn, causal=causal, return_lse=True, out=o, balance=balance)
+        assert res.data_ptr() == o.data_ptr()
+        outs.append((res.clone(), lse.clone()))
+    torch.cuda.synchronize()
+    assert not torch.isnan(outs[1][0]).any()
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][1], outs[1][1])
