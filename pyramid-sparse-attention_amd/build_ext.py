@@ -24,6 +24,14 @@ FLAGS = [
 ]
 
 
+# Per-file additions.  The forward kernel never produces a NaN on purpose (empty rows are handled by
+# explicit -inf tests), and without NaN semantics the row-maximum chains compile to v_max3_f32 without
+# a canonicalising pass over the MFMA results.
+FILE_FLAGS = {
+    "psa_fwd.hip": ["-fno-honor-nans"],
+}
+
+
 def _hipcc():
     for c in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if c and (os.path.isabs(c) and os.path.exists(c) or not os.path.isabs(c)):
@@ -47,7 +55,7 @@ def build(verbose=True, extra_flags=(), out=OUT):
 
     def one(pair):
         s, o = pair
-        out = _run([hipcc, *FLAGS, *extra_flags, "-c", s, "-o", o])
+        out = _run([hipcc, *FLAGS, *FILE_FLAGS.get(os.path.basename(s), []), *extra_flags, "-c", s, "-o", o])
         if verbose and out.strip():
             print(out)
         return o

@@ -25,7 +25,10 @@
 //    reads run one MFMA step ahead.  Two workgroups per CU overlap one's softmax with the other's MFMAs.
 //
 // Roofline: MFMA-bound; 4*BM*64*D flops per tile.
+#include <type_traits>
+
 #include "psa_common.h"
+#include "psa_tiles.h"
 
 namespace {
 
@@ -477,6 +480,328 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   }
 }
 
+// =========================================================================================================
+// Head dim 128: tiles go from global memory straight into LDS (no register staging), V is read back with
+// the transposing LDS load.
+//
+//  * K and V tiles are both kept row-major in LDS, 64 rows of 256 bytes, double buffered.  One
+//    global_load_lds_dwordx4 moves 4 rows (64 lanes x 16 bytes land at consecutive LDS addresses).
+//  * Physical row r of a tile stores its 16-byte chunks XOR-swizzled: chunk c sits at position c ^ (r & 15).
+//    The swizzle is applied on the global side (a lane fetches the chunk that belongs at its LDS position),
+//    so it costs nothing, and it makes the 128-bit K reads and the transposing V reads bank-conflict free.
+//  * Inside each group of 16 rows the rows are stored 4x4-transposed (physical 4n + q holds tile slot
+//    4q + n): the 4 rows a lane fetches are then 4 CONSECUTIVE tile slots, which always belong to one
+//    kv-block, so one block-list lookup per lane and tile serves K and V.
+//  * ds_read_b64_tr_b16 hands every lane 4 keys of one channel from row-major V: exactly the A operand
+//    of O^T += V^T P^T, in the key order that the S^T accumulator layout gives P^T.
+//  * The tile loop is unrolled by two so that the LDS buffer offsets are immediates.
+constexpr int F_TILE = 64 * 256;  // bytes of one K or V tile (D = 128)
+
+#define PSA_LDS(T) __attribute__((address_space(3))) T*
+
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
+  constexpr int D = 128, NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
+  constexpr int G16 = 4 / NW;  // 16-row groups of a tile fetched by one wave
+  constexpr int OST = D * 2 + 16;
+  static_assert(NW == 4 || NW == 2 || NW == 1, "1, 2 or 4 waves");
+  static_assert(BM * OST <= 4 * F_TILE, "O staging must fit the tile buffers");
+  const auto P_L = p.L;
+  const auto P_bn_log2 = p.bn_log2;
+  const auto P_causal = p.causal;
+  const auto P_scale_log2 = p.scale_log2;
+  const auto P_npad = p.npad;
+  const auto P_kp = p.kp;
+  const auto P_vp = p.vp;
+  const uint32_t P_k_strb = (uint32_t)p.k_sl * 2u, P_v_strb = (uint32_t)p.v_sl * 2u;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  // K buffers at 0 and F_TILE, V buffers at 2*F_TILE and 3*F_TILE
+  u32x2* tdesc = (u32x2*)(smem + 4 * F_TILE);
+  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
+
+  const int bid = blockIdx.x;
+  int logical = (bid & 7) * p.wg_chunk + (bid >> 3);
+  if (p.order != nullptr) logical = p.order[logical];
+  if (logical < 0 || logical >= p.total_wg) return;
+  const int I = logical % p.Mq;
+  const int bh = logical / p.Mq;
+  const int h = bh % p.Hq, b = bh / p.Hq;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+
+  int jmax = p.Nk;
+  if (P_causal) {
+    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << P_bn_log2) - 1) >> P_bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  // Q fragments (B operand of S^T = K Q^T): lane holds Q[row l32][16*kk + 8*hh .. +8]
+  const int q_row0 = I * BM + wave * 32;
+  const int q_idx = q_row0 + l32;
+  bf16x8 qf[KK];
+  {
+    const int qr = q_idx < P_L ? q_idx : P_L - 1;
+    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
+  }
+  const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2,
+                                                 P_L, P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff);
+
+  const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
+  const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
+
+  // ---- lane-invariant addressing --------------------------------------------------------------------
+  // fetch: lane (q = lane/16, pos = lane%16) of the n-th instruction of a 16-row group writes physical row
+  // 4n + q, position pos, i.e. tile slot 4q + n, chunk pos ^ (4n + q)
+  const int fq = lane >> 4, fpos = lane & 15;
+  uint32_t f_chunk[4];
+#pragma unroll
+  for (int n = 0; n < 4; ++n) f_chunk[n] = (uint32_t)((fpos ^ fq ^ (4 * n)) * 16);
+  // K operand: tile slot l32 (+32) -> physical row 16*(l32>>4) + 4*(l32&3) + ((l32>>2)&3)
+  uint32_t k_off[KK];
+  {
+    const int fr = 4 * (l32 & 3) + ((l32 >> 2) & 3);
+    const int prow = 16 * (l32 >> 4) + fr;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) k_off[kk] = (uint32_t)(prow * 256 + (((2 * kk + hh) ^ fr) * 16));
+  }
+  // V operand (transposing read).  Inside a block of 16 lanes, lane i supplies the address of 4 channels
+  // (4*(i%4)..) of key i/4 and receives channel i of the block's 4 keys.  Block bl covers channels
+  // 32*db + 16*(bl&1).. and keys 16*cg + 8*s + 4*(bl>>1)..  (s = first / second half of the operand).
+  uint32_t v_off[2][DB];
+  {
+    const int i16 = lane & 15, bl = lane >> 4;
+    const int n = i16 >> 2, bhalf = bl >> 1;
+    const int cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int qq = 2 * s + bhalf;  // tile slot 16*cg + 4*qq + n -> physical row 16*cg + 4*n + qq
+        v_off[s][db] = (uint32_t)((4 * n + qq) * 256 + (((db ^ n) * 4 + (cl ^ qq)) * 16) + hb * 8);
+      }
+  }
+
+  auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
+    const u32x2 dd = tdesc[t];
+    const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd[0]);
+    const uint32_t d1 = __builtin_amdgcn_readfirstlane(dd[1]);
+    const int lv = d0 & 3, nvalid = (d0 >> 3) & 127, lt = d0 >> 10;
+    const int cnt = d1 >> 16;
+    const uint16_t* lids = ids + (d1 & 0xffff);
+    const int sbs_log2 = P_bn_log2 - lv;
+    const int lm1 = lv > 0 ? lv - 1 : 0;
+    const int64_t pool_off = (BHkv * (P_npad - (P_npad >> lm1)) + bhk * (P_npad >> lv)) * (D * 2);
+    const char* kbase = lv == 0 ? kb0 : (const char*)P_kp + pool_off;
+    const char* vbase = lv == 0 ? vb0 : (const char*)P_vp + pool_off;
+    const uint32_t kstr = lv == 0 ? P_k_strb : (uint32_t)(D * 2);
+    const uint32_t vstr = lv == 0 ? P_v_strb : (uint32_t)(D * 2);
+    const bool ragged = nvalid < TK;  // some slots are empty: clamp them onto real rows (their logits are masked)
+    const int row_lim = lv == 0 ? P_L - 1 : 0x7fffffff;
+#pragma unroll
+    for (int gi = 0; gi < G16; ++gi) {
+      const int g16 = wave * G16 + gi;
+      const int g = (lt << 6) + g16 * 16 + fq * 4;
+      int bi = g >> sbs_log2;
+      if (ragged) bi = bi < cnt - 1 ? bi : cnt - 1;
+      const int src0 = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        int src = src0 + n;
+        if (ragged) src = src < row_lim ? src : row_lim;
+        const uint32_t ko = (uint32_t)src * kstr + f_chunk[n];
+        const uint32_t vo = (uint32_t)src * vstr + f_chunk[n];
+        const int dst = buf * F_TILE + (g16 * 4 + n) * 1024;
+        __builtin_amdgcn_global_load_lds(kbase + ko, (PSA_LDS(void))(smem + dst), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(vbase + vo, (PSA_LDS(void))(smem + 2 * F_TILE + dst), 16, 0, 0);
+      }
+    }
+  };
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  float m_run = -INFINITY;  // running reference max (log2 domain), same in both half-waves
+  float l_run = 0.f;        // this lane's partial row sum
+
+  auto compute_tile = [&](int t, auto buf_c) __attribute__((always_inline)) {
+    constexpr int BUF = decltype(buf_c)::value;
+    const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
+    const int lv = d & 3;
+    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + BUF * F_TILE;
+    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + BUF) * F_TILE;
+    f32x16 s_cur[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_cur[c][i] = 0.f;
+    {
+      bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 32 * 256);
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        bf16x8 n0 = a0, n1 = a1;
+        if (kk + 1 < KK) {
+          n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[kk + 1]);
+          n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[kk + 1] + 32 * 256);
+        }
+        s_cur[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s_cur[0], 0, 0, 0);
+        s_cur[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s_cur[1], 0, 0, 0);
+        a0 = n0;
+        a1 = n1;
+      }
+    }
+
+    if (d & 4) {  // partly empty tile and/or causal diagonal: mask individual keys
+      const psa_tiles::TileRef r = psa_tiles::tile_ref(tdesc, ids, t, P_bn_log2);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int r0 = c * 32 + g * 8 + hh * 4;
+          int src0 = -1;
+          if (r0 < r.nvalid) src0 = psa_tiles::slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool in_tile = src0 >= 0 && (r0 + e) < r.nvalid;
+            // causal: a pooled key is visible once its last constituent token is
+            const bool visible = !P_causal || ((((int64_t)(src0 + e) + 1) << lv) - 1 <= (int64_t)q_idx);
+            const float sv = s_cur[c][g * 4 + e];
+            s_cur[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
+          }
+        }
+    }
+
+    // online softmax of tile t (per query column = per lane, both half-waves)
+    float mx0 = s_cur[0][0], mx1 = s_cur[1][0];
+#pragma unroll
+    for (int i = 1; i < 15; i += 2) {
+      mx0 = max3(mx0, s_cur[0][i], s_cur[0][i + 1]);
+      mx1 = max3(mx1, s_cur[1][i], s_cur[1][i + 1]);
+    }
+    float mx = max3(mx0, s_cur[0][15], max3(mx1, s_cur[1][15], -INFINITY));
+    mx = fmaxf(mx, shfl_xor32(mx));
+    const float bias = (float)lv;
+    const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
+    // raise the reference max only when it lags by more than the threshold (or is still -inf)
+    float m_new = (m_cand - m_run > LAZY_THRESHOLD) ? m_cand : m_run;
+    m_new = (m_run == -INFINITY) ? m_cand : m_new;
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that still see no key
+    const float alpha = fast_exp2(m_run - m_use);
+    const float nb = bias - m_use;
+    uint32_t pk[2][8];
+    float lsum = 0.f;
+    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = fast_exp2(__builtin_fmaf(s_cur[c][i], P_scale_log2, nb));
+        const float p1 = fast_exp2(__builtin_fmaf(s_cur[c][i + 1], P_scale_log2, nb));
+        pk[c][i >> 1] = pack_bf16x2(p0, p1);
+        // row sum of the ROUNDED probabilities (the same values that multiply V)
+        lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[c][i >> 1]), ones, lsum, false);
+      }
+    }
+    l_run = l_run * alpha + lsum;
+    m_run = m_new;
+
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+    }
+
+    // O^T += V^T P^T : per 16-key group cg, A = V^T[32 d][16 keys] (two transposing reads), B = P^T
+    u32x2 vlo[DB], vhi[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      vlo[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0][db])));
+      vhi[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1][db])));
+    }
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg) {
+      const int c = cg >> 1, g = cg & 1;
+      u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
+      const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
+      u32x2 nlo[DB], nhi[DB];
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        nlo[db] = vlo[db];
+        nhi[db] = vhi[db];
+        if (cg + 1 < 4) {
+          nlo[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0][db] + (cg + 1) * 4096)));
+          nhi[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1][db] + (cg + 1) * 4096)));
+        }
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        u32x4 aw = {vlo[db][0], vlo[db][1], vhi[db][0], vhi[db][1]};
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        vlo[db] = nlo[db];
+        vhi[db] = nhi[db];
+      }
+    }
+  };
+
+  if (T > 0) {
+    issue_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the tile has landed in LDS
+    __syncthreads();
+    for (int t = 0; t < T; t += 2) {
+      // invariant: LDS buffers (t & 1) hold tile t; the other pair is free
+      if (t + 1 < T) issue_tile(t + 1, 1);
+      compute_tile(t, std::integral_constant<int, 0>{});
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      if (t + 1 < T) {
+        if (t + 2 < T) issue_tile(t + 2, 0);
+        compute_tile(t + 1, std::integral_constant<int, 1>{});
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+      }
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------
+  float l_tot = l_run + shfl_xor32(l_run);
+  const float l_safe = fmaxf(l_tot, 1e-8f);
+  const float inv = 1.0f / l_safe;
+  if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
+    // natural-log domain: m*ln2 + ln(max(l, 1e-8))
+    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+  }
+  __syncthreads();  // everyone is done with the last K/V tile
+  unsigned char* Os = smem;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
+      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
+      *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
+    }
+  __syncthreads();
+  bf16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
+  for (int u = tid; u < BM * CH; u += NT) {
+    const int r = u / CH, ch = u % CH;
+    const int row = I * BM + r;
+    if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+  }
+}
+
 // ---- longest-rows-first ordering ---------------------------------------------------------------------
 // Rows of the level map differ in the number of tiles they retain.  Workgroup ids are dealt round-robin
 // to the 8 XCDs and each XCD runs its ids in order, so sorting every XCD's share by decreasing tile count
@@ -548,6 +873,16 @@ int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   return PSA_OK;
 }
 
+template <int NW>
+int launch_fwd_d128(const FwdParams& p, int Nk, hipStream_t stream) {
+  size_t shmem = (size_t)4 * F_TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
+  if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
+  if (hipFuncSetAttribute((const void*)psa_fwd_d128_kernel<NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+    return PSA_ERR_LAUNCH;
+  hipLaunchKernelGGL((psa_fwd_d128_kernel<NW>), dim3((unsigned)(p.wg_chunk * 8)), dim3(NW * 64), shmem, stream, p);
+  return PSA_OK;
+}
+
 }  // namespace
 
 extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
@@ -608,8 +943,8 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     p.order = order;
   }
   int rc;
-  if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
-  else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);
+  if (D == 128 && block_m == 128) rc = launch_fwd_d128<4>(p, Nk, (hipStream_t)stream);
+  else if (D == 128) rc = launch_fwd_d128<2>(p, Nk, (hipStream_t)stream);
   else if (block_m == 128) rc = launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
   else rc = launch_fwd<64, 2>(p, Nk, (hipStream_t)stream);
   PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");
