@@ -65,9 +65,24 @@ __device__ __forceinline__ float max3f(float a, float b, float c) {
   return r;
 }
 
-__device__ __forceinline__ float shfl_xor32(float v) {
-  // exchange between the two 32-lane halves of a wave
-  return __shfl_xor(v, 32, 64);
+// Exchange between the two 32-lane halves of a wave (v_permlane32_swap: no LDS round trip).
+// After the swap r[0] holds lanes 0-31 of v in both halves and r[1] holds lanes 32-63 in both halves.
+__device__ __forceinline__ void half_wave_swap(float v, float& lo, float& hi) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];  // element-wise extraction first: a bit_cast of r[i] itself reads element 0
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float half_wave_max(float v) {
+  float lo, hi;
+  half_wave_swap(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+  float lo, hi;
+  half_wave_swap(v, lo, hi);
+  return lo + hi;
 }
 
 // level value (0,1,2,4,8) of a map element of 1 or 4 bytes

@@ -158,19 +158,19 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_est_gemm_kernel(EstParams p) {
       const int jbase = (t * 2 + c) << gpc_log2;
       if (gpc_log2 == 0) {
         float v = fmaxf(fmaxf(o4[0], o4[1]), fmaxf(o4[2], o4[3]));
-        v = fmaxf(v, shfl_xor32(v)) * qk_scale;
+        v = half_wave_max(v) * qk_scale;
         m_run = fmaxf(m_run, v);
         if (hh == 0) rt[(int64_t)jbase * rts] = v;
       } else if (gpc_log2 == 1) {
         float v0 = fmaxf(o4[0], o4[1]), v1 = fmaxf(o4[2], o4[3]);
-        v0 = fmaxf(v0, shfl_xor32(v0)) * qk_scale;
-        v1 = fmaxf(v1, shfl_xor32(v1)) * qk_scale;
+        v0 = half_wave_max(v0) * qk_scale;
+        v1 = half_wave_max(v1) * qk_scale;
         m_run = fmaxf(m_run, fmaxf(v0, v1));
         rt[(int64_t)(jbase + hh) * rts] = hh ? v1 : v0;
       } else {
 #pragma unroll
         for (int o = 0; o < 4; ++o) {
-          const float v = fmaxf(o4[o], shfl_xor32(o4[o])) * qk_scale;
+          const float v = half_wave_max(o4[o]) * qk_scale;
           m_run = fmaxf(m_run, v);
           if ((o & 1) == hh) rt[(int64_t)(jbase + o) * rts] = v;
         }

@@ -381,7 +381,7 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
       float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
 #pragma unroll
       for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s_cur[0][i], s_cur[1][i]));
-      mx = fmaxf(mx, shfl_xor32(mx));
+      mx = half_wave_max(mx);
       const float bias = (float)lv;
       const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
       // raise the reference max only when it lags by more than the threshold (or is still -inf)
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   }
 
   // ---- 5. epilogue --------------------------------------------------------------------------
-  float l_tot = l_run + shfl_xor32(l_run);
+  float l_tot = half_wave_sum(l_run);
   const float l_safe = fmaxf(l_tot, 1e-8f);
   const float inv = 1.0f / l_safe;
   if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
@@ -482,24 +482,33 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
 
 // =========================================================================================================
 // Head dim 128: tiles go from global memory straight into LDS (no register staging), V is read back with
-// the transposing LDS load.
+// the transposing LDS load, and the exponentials of one tile overlap the QK^T MFMAs of the next.
 //
-//  * K and V tiles are both kept row-major in LDS, 64 rows of 256 bytes, double buffered.  One
-//    global_load_lds_dwordx4 moves 4 rows (64 lanes x 16 bytes land at consecutive LDS addresses).
-//  * Physical row r of a tile stores its 16-byte chunks XOR-swizzled: chunk c sits at position c ^ (r & 15).
-//    The swizzle is applied on the global side (a lane fetches the chunk that belongs at its LDS position),
-//    so it costs nothing, and it makes the 128-bit K reads and the transposing V reads bank-conflict free.
-//  * Inside each group of 16 rows the rows are stored 4x4-transposed (physical 4n + q holds tile slot
+//  * K and V tiles are both kept row-major in LDS, double buffered.  One global_load_lds_dwordx4 moves 4
+//    rows of 256 bytes (64 lanes x 16 bytes land at consecutive LDS addresses); the 16 four-row blocks of
+//    a tile are F_ISTR = 1024 + 64 bytes apart, and row q of a block stores its 16-byte chunks
+//    XOR-swizzled: chunk c sits at position c ^ q.  The swizzle is applied on the global side (a lane
+//    fetches the chunk that belongs at its LDS position), so it costs nothing.  Padding and swizzle together
+//    make the 128-bit K reads and the transposing V reads bank-conflict free, and both only touch the low
+//    bits of the chunk index, so every operand address is lane base + immediate.
+//  * Inside each group of 16 rows the rows are stored 4x4-transposed (block n, row q holds tile slot
 //    4q + n): the 4 rows a lane fetches are then 4 CONSECUTIVE tile slots, which always belong to one
 //    kv-block, so one block-list lookup per lane and tile serves K and V.
 //  * ds_read_b64_tr_b16 hands every lane 4 keys of one channel from row-major V: exactly the A operand
 //    of O^T += V^T P^T, in the key order that the S^T accumulator layout gives P^T.
 //  * The tile loop is unrolled by two so that the LDS buffer offsets are immediates.
-constexpr int F_TILE = 64 * 256;  // bytes of one K or V tile (D = 128)
+constexpr int F_ISTR = 1024 + 64;     // bytes between the 4-row blocks of a tile
+constexpr int F_TILE = 16 * F_ISTR;   // bytes of one K or V tile (D = 128)
 
 #define PSA_LDS(T) __attribute__((address_space(3))) T*
 
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
+#define TILE_SYNC()                         \
+  do {                                      \
+    __builtin_amdgcn_s_waitcnt(0x0f70);     \
+    __syncthreads();                        \
+  } while (0)
 
 template <int NW>
 __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
@@ -531,7 +540,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   const int bh = logical / p.Mq;
   const int h = bh % p.Hq, b = bh / p.Hq;
   const int hk = h / (p.Hq / p.Hkv);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hh = lane >> 5;
 
   int jmax = p.Nk;
@@ -557,38 +566,44 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
 
   // ---- lane-invariant addressing --------------------------------------------------------------------
-  // fetch: lane (q = lane/16, pos = lane%16) of the n-th instruction of a 16-row group writes physical row
-  // 4n + q, position pos, i.e. tile slot 4q + n, chunk pos ^ (4n + q)
-  const int fq = lane >> 4, fpos = lane & 15;
-  uint32_t f_chunk[4];
-#pragma unroll
-  for (int n = 0; n < 4; ++n) f_chunk[n] = (uint32_t)((fpos ^ fq ^ (4 * n)) * 16);
-  // K operand: tile slot l32 (+32) -> physical row 16*(l32>>4) + 4*(l32&3) + ((l32>>2)&3)
-  uint32_t k_off[KK];
+  // fetch: lane (q = lane/16, pos = lane%16) of block n of a 16-row group writes row q of that block at
+  // position pos, i.e. tile slot 4q + n, chunk pos ^ q
+  const int fq = lane >> 4;
+  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
+  // K operand of k-step kk: tile slot l32 (+32) = block 4*(l32>>4) + (l32&3), row (l32>>2)&3, chunk 2kk + hh
+  // -> k_off[kk & 1] + 64 * (kk >> 1)   (+ 8 blocks for the second 32 keys)
+  uint32_t k_off[2];
   {
-    const int fr = 4 * (l32 & 3) + ((l32 >> 2) & 3);
-    const int prow = 16 * (l32 >> 4) + fr;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) k_off[kk] = (uint32_t)(prow * 256 + (((2 * kk + hh) ^ fr) * 16));
+    const int q = (l32 >> 2) & 3;
+    const int base = (4 * (l32 >> 4) + (l32 & 3)) * F_ISTR + q * 256;
+    k_off[0] = (uint32_t)(base + ((hh ^ q) * 16));
+    k_off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
   }
   // V operand (transposing read).  Inside a block of 16 lanes, lane i supplies the address of 4 channels
-  // (4*(i%4)..) of key i/4 and receives channel i of the block's 4 keys.  Block bl covers channels
-  // 32*db + 16*(bl&1).. and keys 16*cg + 8*s + 4*(bl>>1)..  (s = first / second half of the operand).
-  uint32_t v_off[2][DB];
+  // (4*(i%4)..) of key i/4 and receives channel i of the block's 4 keys.  Lane block bl covers channels
+  // 32*db + 16*(bl&1).. and keys 16*cg + 8*s + 4*(bl>>1)..  (s = first / second half of the operand):
+  // tile slot 16*cg + 4*qq + n with qq = 2s + (bl>>1), n = i/4 -> block 4*cg + n, row qq
+  // -> v_off[s] + 64 * db + 4 * F_ISTR * cg
+  uint32_t v_off[2];
   {
     const int i16 = lane & 15, bl = lane >> 4;
-    const int n = i16 >> 2, bhalf = bl >> 1;
-    const int cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
+    const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int qq = 2 * s + bhalf;  // tile slot 16*cg + 4*qq + n -> physical row 16*cg + 4*n + qq
-        v_off[s][db] = (uint32_t)((4 * n + qq) * 256 + (((db ^ n) * 4 + (cl ^ qq)) * 16) + hb * 8);
-      }
+    for (int s = 0; s < 2; ++s) {
+      const int qq = 2 * s + (bl >> 1);
+      v_off[s] = (uint32_t)(n * F_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
+    }
   }
 
-  auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
+  // Where tile t comes from: base pointers and row strides (uniform), and for every 16-row group this
+  // wave fetches the first of the lane's 4 consecutive source rows.
+  struct TileSrc {
+    const char *kbase, *vbase;
+    uint32_t kstr, vstr;
+    int lim;          // last valid row when the tile may run past the sequence end, else INT_MAX
+    int src0[G16];
+  };
+  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) {
     const u32x2 dd = tdesc[t];
     const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd[0]);
     const uint32_t d1 = __builtin_amdgcn_readfirstlane(dd[1]);
@@ -598,28 +613,37 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     const int sbs_log2 = P_bn_log2 - lv;
     const int lm1 = lv > 0 ? lv - 1 : 0;
     const int64_t pool_off = (BHkv * (P_npad - (P_npad >> lm1)) + bhk * (P_npad >> lv)) * (D * 2);
-    const char* kbase = lv == 0 ? kb0 : (const char*)P_kp + pool_off;
-    const char* vbase = lv == 0 ? vb0 : (const char*)P_vp + pool_off;
-    const uint32_t kstr = lv == 0 ? P_k_strb : (uint32_t)(D * 2);
-    const uint32_t vstr = lv == 0 ? P_v_strb : (uint32_t)(D * 2);
+    a.kbase = lv == 0 ? kb0 : (const char*)P_kp + pool_off;
+    a.vbase = lv == 0 ? vb0 : (const char*)P_vp + pool_off;
+    a.kstr = lv == 0 ? P_k_strb : (uint32_t)(D * 2);
+    a.vstr = lv == 0 ? P_v_strb : (uint32_t)(D * 2);
     const bool ragged = nvalid < TK;  // some slots are empty: clamp them onto real rows (their logits are masked)
-    const int row_lim = lv == 0 ? P_L - 1 : 0x7fffffff;
+    a.lim = (ragged && lv == 0) ? P_L - 1 : 0x7fffffff;
 #pragma unroll
     for (int gi = 0; gi < G16; ++gi) {
-      const int g16 = wave * G16 + gi;
-      const int g = (lt << 6) + g16 * 16 + fq * 4;
+      const int g = (lt << 6) + (wave * G16 + gi) * 16 + fq * 4;
       int bi = g >> sbs_log2;
       if (ragged) bi = bi < cnt - 1 ? bi : cnt - 1;
-      const int src0 = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
+      a.src0[gi] = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
+    }
+  };
+  // 4 rows per instruction go to block 4*g16 + n of the buffer at lds_byte
+  auto issue_rows = [&](const char* base, uint32_t str, int lim, const int (&src0)[G16], int lds_byte) __attribute__((always_inline)) {
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
-        int src = src0 + n;
-        if (ragged) src = src < row_lim ? src : row_lim;
-        const uint32_t ko = (uint32_t)src * kstr + f_chunk[n];
-        const uint32_t vo = (uint32_t)src * vstr + f_chunk[n];
-        const int dst = buf * F_TILE + (g16 * 4 + n) * 1024;
-        __builtin_amdgcn_global_load_lds(kbase + ko, (PSA_LDS(void))(smem + dst), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(vbase + vo, (PSA_LDS(void))(smem + 2 * F_TILE + dst), 16, 0, 0);
+    for (int gi = 0; gi < G16; ++gi) {
+      const int blk = (wave * G16 + gi) * 4;
+      if (lim == 0x7fffffff) {
+        // the usual case: the uniform base pointer steps from row to row, the lane offset stays
+        const uint32_t off = (uint32_t)src0[gi] * str + f_chunk;
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+          __builtin_amdgcn_global_load_lds(base + (uint64_t)(n * str) + off, (PSA_LDS(void))(smem + lds_byte + (blk + n) * F_ISTR), 16, 0, 0);
+      } else {
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+          const int src = src0[gi] + n < lim ? src0[gi] + n : lim;
+          __builtin_amdgcn_global_load_lds(base + ((uint32_t)src * str + f_chunk), (PSA_LDS(void))(smem + lds_byte + (blk + n) * F_ISTR), 16, 0, 0);
+        }
       }
     }
   };
@@ -631,151 +655,171 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
   float m_run = -INFINITY;  // running reference max (log2 domain), same in both half-waves
   float l_run = 0.f;        // this lane's partial row sum
+  const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
 
-  auto compute_tile = [&](int t, auto buf_c) __attribute__((always_inline)) {
-    constexpr int BUF = decltype(buf_c)::value;
+  // masks (if needed) and reduces the logits of tile t; returns the bias - reference max and the rescale factor
+  auto softmax_head = [&](int t, f32x16 (&s_cur)[2], float& nb, float& alpha) __attribute__((always_inline)) {
     const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
     const int lv = d & 3;
-    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + BUF * F_TILE;
-    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + BUF) * F_TILE;
-    f32x16 s_cur[2];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_cur[c][i] = 0.f;
-    {
-      bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 32 * 256);
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        bf16x8 n0 = a0, n1 = a1;
-        if (kk + 1 < KK) {
-          n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[kk + 1]);
-          n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[kk + 1] + 32 * 256);
-        }
-        s_cur[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s_cur[0], 0, 0, 0);
-        s_cur[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s_cur[1], 0, 0, 0);
-        a0 = n0;
-        a1 = n1;
-      }
-    }
-
-    if (d & 4) {  // partly empty tile and/or causal diagonal: mask individual keys
-      const psa_tiles::TileRef r = psa_tiles::tile_ref(tdesc, ids, t, P_bn_log2);
+    if (d & 4) {
+      // Partly empty tile and/or causal diagonal.  Valid slots are a prefix of the tile (nvalid), and a
+      // pooled key of level lv is visible to query i once its last token is: ((src + 1) << lv) - 1 <= i, i.e.
+      // src < (i + 1) >> lv.  Both limits cut each run of 4 consecutive slots after its first `keep` elements.
+      const int nvalid = (int)((d >> 3) & 127);
+      const int qlim = (q_idx + 1) >> lv;
+      const uint32_t d1 = __builtin_amdgcn_readfirstlane(tdesc[t][1]);
+      const int cnt = (int)(d1 >> 16), lt = (int)(d >> 10), sbs_log2 = P_bn_log2 - lv;
+      const uint16_t* lids = ids + (d1 & 0xffff);
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int r0 = c * 32 + g * 8 + hh * 4;
-          int src0 = -1;
-          if (r0 < r.nvalid) src0 = psa_tiles::slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const bool in_tile = src0 >= 0 && (r0 + e) < r.nvalid;
-            // causal: a pooled key is visible once its last constituent token is
-            const bool visible = !P_causal || ((((int64_t)(src0 + e) + 1) << lv) - 1 <= (int64_t)q_idx);
-            const float sv = s_cur[c][g * 4 + e];
-            s_cur[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
+          int keep = nvalid - r0;
+          if (P_causal) {
+            const int gpos = (lt << 6) + r0;
+            int bi = gpos >> sbs_log2;
+            bi = bi < cnt - 1 ? bi : cnt - 1;
+            const int src0 = ((int)lids[bi] << sbs_log2) + (gpos & ((1 << sbs_log2) - 1));
+            keep = keep < qlim - src0 ? keep : qlim - src0;
           }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s_cur[c][g * 4 + e] = e < keep ? s_cur[c][g * 4 + e] : -INFINITY;
         }
     }
-
-    // online softmax of tile t (per query column = per lane, both half-waves)
     float mx0 = s_cur[0][0], mx1 = s_cur[1][0];
 #pragma unroll
     for (int i = 1; i < 15; i += 2) {
       mx0 = max3(mx0, s_cur[0][i], s_cur[0][i + 1]);
       mx1 = max3(mx1, s_cur[1][i], s_cur[1][i + 1]);
     }
-    float mx = max3(mx0, s_cur[0][15], max3(mx1, s_cur[1][15], -INFINITY));
-    mx = fmaxf(mx, shfl_xor32(mx));
+    float mx = max3(mx0, s_cur[0][15], fmaxf(mx1, s_cur[1][15]));
+    mx = half_wave_max(mx);
     const float bias = (float)lv;
     const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
     // raise the reference max only when it lags by more than the threshold (or is still -inf)
     float m_new = (m_cand - m_run > LAZY_THRESHOLD) ? m_cand : m_run;
     m_new = (m_run == -INFINITY) ? m_cand : m_new;
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that still see no key
-    const float alpha = fast_exp2(m_run - m_use);
-    const float nb = bias - m_use;
-    uint32_t pk[2][8];
-    float lsum = 0.f;
-    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        const float p0 = fast_exp2(__builtin_fmaf(s_cur[c][i], P_scale_log2, nb));
-        const float p1 = fast_exp2(__builtin_fmaf(s_cur[c][i + 1], P_scale_log2, nb));
-        pk[c][i >> 1] = pack_bf16x2(p0, p1);
-        // row sum of the ROUNDED probabilities (the same values that multiply V)
-        lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[c][i >> 1]), ones, lsum, false);
-      }
-    }
-    l_run = l_run * alpha + lsum;
+    alpha = fast_exp2(m_run - m_use);
+    nb = bias - m_use;
     m_run = m_new;
-
+  };
+  // probabilities of 4 logits: exp2, round to bf16, add the ROUNDED values (the ones that multiply V) to the row sum
+  auto prob4 = [&](const f32x16& sc, int i, float nb, uint32_t* pk2, float& lsum) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 4; e += 2) {
+      const float p0 = fast_exp2(__builtin_fmaf(sc[i + e], P_scale_log2, nb));
+      const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb));
+      pk2[e >> 1] = pack_bf16x2(p0, p1);
+      lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk2[e >> 1]), ones, lsum, false);
+    }
+  };
+  // exponentials of the 16 logits of one 32-key half (4 groups of 4)
+  auto prob16 = [&](const f32x16& sc, float nb, uint32_t* pk8, float& lsum) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) prob4(sc, i * 4, nb, pk8 + i * 2, lsum);
+  };
+  // Both halves of S^T at once: two independent accumulation chains, operands fetched one k-step ahead.
+  auto qk_full = [&](auto kb_c, f32x16 (&s2)[2]) __attribute__((always_inline)) {
+    constexpr int KB = decltype(kb_c)::value;
+    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + KB * F_TILE;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s2[c][i] = 0.f;
+    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 8 * F_ISTR);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      bf16x8 n0 = a0, n1 = a1;
+      if (kk + 1 < KK) {
+        n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
+        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + 8 * F_ISTR);
+      }
+      s2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s2[0], 0, 0, 0);
+      s2[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s2[1], 0, 0, 0);
+      a0 = n0;
+      a1 = n1;
+    }
+  };
+  // Half hf (32 keys) of O^T += V^T P^T from V buffer VB: per 16-key group cg, A = V^T[32 d][16 keys] (two
+  // transposing reads), B = P^T.  8 MFMAs on 4 independent accumulators.
+  auto pv_half = [&](auto vb_c, int hf, const uint32_t* pk8) __attribute__((always_inline)) {
+    constexpr int VB = decltype(vb_c)::value;
+    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + VB) * F_TILE + hf * (8 * F_ISTR);
+    // operand of MFMA step st = 4*g + db; reads run AHEAD steps in front of the MFMAs
+    constexpr int AHEAD = 2, STEPS = 2 * DB;
+    auto vread = [&](int st, int s) __attribute__((always_inline)) {
+      return __builtin_bit_cast(
+          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[s] + (st & 3) * 64 + (st >> 2) * (4 * F_ISTR))));
+    };
+    u32x2 vlo[STEPS], vhi[STEPS];  // fully unrolled: every element is a short-lived register value
+#pragma unroll
+    for (int st = 0; st < AHEAD; ++st) {
+      vlo[st] = vread(st, 0);
+      vhi[st] = vread(st, 1);
+    }
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const int g = st >> 2, db = st & 3;
+      if (st + AHEAD < STEPS) {
+        vlo[st + AHEAD] = vread(st + AHEAD, 0);
+        vhi[st + AHEAD] = vread(st + AHEAD, 1);
+      }
+      u32x4 bw = {pk8[g * 4 + 0], pk8[g * 4 + 1], pk8[g * 4 + 2], pk8[g * 4 + 3]};
+      u32x4 aw = {vlo[st][0], vlo[st][1], vhi[st][0], vhi[st][1]};
+      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), __builtin_bit_cast(bf16x8, bw), acc[db], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads AHEAD steps in front, not more
+    }
+  };
+  auto rescale_acc = [&](float alpha) __attribute__((always_inline)) {
     if (__any(alpha != 1.0f)) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
     }
-
-    // O^T += V^T P^T : per 16-key group cg, A = V^T[32 d][16 keys] (two transposing reads), B = P^T
-    u32x2 vlo[DB], vhi[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      vlo[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0][db])));
-      vhi[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1][db])));
-    }
-#pragma unroll
-    for (int cg = 0; cg < 4; ++cg) {
-      const int c = cg >> 1, g = cg & 1;
-      u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
-      const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
-      u32x2 nlo[DB], nhi[DB];
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        nlo[db] = vlo[db];
-        nhi[db] = vhi[db];
-        if (cg + 1 < 4) {
-          nlo[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0][db] + (cg + 1) * 4096)));
-          nhi[db] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1][db] + (cg + 1) * 4096)));
-        }
-      }
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        u32x4 aw = {vlo[db][0], vlo[db][1], vhi[db][0], vhi[db][1]};
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
-      }
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        vlo[db] = nlo[db];
-        vhi[db] = nhi[db];
-      }
-    }
   };
+  const std::integral_constant<int, 0> B0;
+  const std::integral_constant<int, 1> B1;
 
+  // Per tile: DMA tile t+1 | QK(t) | softmax(t) | PV(t) | barrier.  The MFMA phases of one workgroup overlap
+  // the softmax of the other workgroup on the CU.  (Interleaving the exponentials of tile t with the MFMAs of
+  // tiles t-1 / t+1 inside one wave was measured and is slower: it serialises the MFMA chains and costs registers.)
   if (T > 0) {
-    issue_tile(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the tile has landed in LDS
-    __syncthreads();
-    for (int t = 0; t < T; t += 2) {
-      // invariant: LDS buffers (t & 1) hold tile t; the other pair is free
-      if (t + 1 < T) issue_tile(t + 1, 1);
-      compute_tile(t, std::integral_constant<int, 0>{});
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      __syncthreads();
+    TileSrc ts;
+    f32x16 s[2];
+    uint32_t pk[2][8];
+    tile_src(0, ts);
+    issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, 0);
+    issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, 2 * F_TILE);
+    TILE_SYNC();
+    auto step = [&](int t, auto cur_c) __attribute__((always_inline)) {
+      constexpr int CUR = decltype(cur_c)::value;
       if (t + 1 < T) {
-        if (t + 2 < T) issue_tile(t + 2, 0);
-        compute_tile(t + 1, std::integral_constant<int, 1>{});
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        __syncthreads();
+        tile_src(t + 1, ts);
+        issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, (CUR ^ 1) * F_TILE);
+        issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, (2 + (CUR ^ 1)) * F_TILE);
       }
+      float nb, alpha, lsum = 0.f;
+      qk_full(cur_c, s);
+      softmax_head(t, s, nb, alpha);
+      prob16(s[0], nb, pk[0], lsum);
+      prob16(s[1], nb, pk[1], lsum);
+      l_run = l_run * alpha + lsum;
+      rescale_acc(alpha);
+      pv_half(cur_c, 0, pk[0]);
+      pv_half(cur_c, 1, pk[1]);
+      TILE_SYNC();
+    };
+    for (int t = 0; t < T; t += 2) {
+      step(t, B0);
+      if (t + 1 < T) step(t + 1, B1);
     }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
-  float l_tot = l_run + shfl_xor32(l_run);
+  float l_tot = half_wave_sum(l_run);
   const float l_safe = fmaxf(l_tot, 1e-8f);
   const float inv = 1.0f / l_safe;
   if (p.lse != nullptr && hh == 0 && q_idx < P_L) {

@@ -135,12 +135,12 @@ __global__ __launch_bounds__(256, 2) void psa_xattn_gemm_kernel(XParams p) {
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 4 * OPB; ++i) mx = fmaxf(mx, z[blk * 4 * OPB + i]);
-        mx = fmaxf(mx, shfl_xor32(mx));
+        mx = half_wave_max(mx);
         const float ref = mx == -INFINITY ? 0.f : mx;
         float sm = 0.f;
 #pragma unroll
         for (int i = 0; i < 4 * OPB; ++i) sm += fast_exp2(z[blk * 4 * OPB + i] - ref);
-        sm += shfl_xor32(sm);
+        sm = half_wave_sum(sm);
         if (hh == 0) {
           const int J = (nb0 + blk * 8 * OPB) >> RBL;
           f32x2 pr = {mx, sm};
