@@ -63,6 +63,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention comparison legs (keeps kernel profiles clean)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="after the run, stream 1 GiB through a plain elementwise kernel (reads 1 GiB, writes 1 GiB): "
+                         "under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its reading calibrates the counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by (batch, head) with no exchange, "
@@ -147,7 +150,7 @@ def main():
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
 
     roofline = {
-        "kernel": "psa_fwd_kernel",
+        "kernel": "psa_fwd_d128_kernel" if D == 128 else "psa_fwd_kernel",
         "bound": "mfma",
         "achieved": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12, 2),
         "peak": PEAK_BF16_TFLOPS,
@@ -189,6 +192,14 @@ def main():
             "sample": "heads %s of %d in fp32: full estimate + level map, attention on %d of %d q-blocks scaled to all; "
                       "then scaled by H/%d" % (heads, H, len(qblocks), Mq, len(heads)),
         }
+
+    if args.copy_calib:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     eff_tflops = dense_flops / (ms_step * 1e-3) / 1e12
     line = {

@@ -24,11 +24,12 @@ FLAGS = [
 ]
 
 
-# Per-file additions.  The forward kernel never produces a NaN on purpose (empty rows are handled by
-# explicit -inf tests), and without NaN semantics the row-maximum chains compile to v_max3_f32 without
-# a canonicalising pass over the MFMA results.
+# Per-file additions.  These kernels never produce a NaN on purpose (empty rows are handled by explicit
+# -inf tests), and without NaN semantics their maximum chains compile to v_max3_f32 without a
+# canonicalising pass over the MFMA results.
 FILE_FLAGS = {
     "psa_fwd.hip": ["-fno-honor-nans"],
+    "psa_estimate.hip": ["-fno-honor-nans"],
 }
 
 

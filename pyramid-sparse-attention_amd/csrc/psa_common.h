@@ -56,14 +56,10 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// v_max3_f32.  The compiler does not track hazards for inline assembly: never feed it a value that an
-// MFMA instruction has just produced (the required wait states are only inserted for instructions
-// the compiler knows); values that went through another VALU op, or are a loop iteration old, are fine.
-__device__ __forceinline__ float max3f(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
+// max of three: compiles to one v_max3_f32 in translation units built without NaN semantics (the compiler then
+// needs no canonicalising pass over its inputs).  Plain C on purpose: hand-written assembly would not get the
+// wait states that reading a fresh MFMA result requires.
+__device__ __forceinline__ float max3f(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
 // Exchange between the two 32-lane halves of a wave (v_permlane32_swap: no LDS round trip).
 // After the swap r[0] holds lanes 0-31 of v in both halves and r[1] holds lanes 32-63 in both halves.

@@ -18,13 +18,15 @@
 namespace {
 
 constexpr int TK = 64;
+constexpr int EST_MAX_KSPLIT = 4;
 
 struct EstParams {
   const bf16_t *q, *k;
   int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl;
   const int32_t *off_q, *off_k;
   float* rt;   // workspace: R^T [B*Hq][n_d][Ms_pad]
-  float* mrow; // workspace: m [B*Hq][Ms_pad]
+  float* mrow; // workspace: m [B*Hq][ksplit][Ms_pad]: row maxima over each share of the keys
+  int ksplit;  // the key range is cut into ksplit shares (grid z) to even out the load
   float* scores;
   int Hq, Hkv, Lq, Lk;
   int bm, bn, keep_m_log2, keep_n_log2;
@@ -178,7 +180,199 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_est_gemm_kernel(EstParams p) {
     }
     __syncthreads();
   }
-  if (hh == 0) p.mrow[(int64_t)bh * p.Ms_pad + row0 + l32] = m_run;
+  if (hh == 0) p.mrow[(int64_t)bh * p.ksplit * p.Ms_pad + row0 + l32] = m_run;
+}
+
+// Head dim 128: 64 sampled query rows per wave (two B-operand sets share every K operand fetched from LDS)
+// and K tiles copied from global memory straight into LDS, double buffered.
+//
+// LDS tile layout (shared with the attention forward kernel): a tile is 16 blocks of 4 rows x 256 bytes, blocks
+// E_ISTR = 1024 + 64 bytes apart; block n, row q of a 16-row group holds tile slot 4q + n, with its 16-byte
+// chunks XOR-swizzled by q.  One global_load_lds_dwordx4 fills one block; the 128-bit operand reads are bank
+// conflict free and their addresses are lane base + immediate.
+constexpr int E_ISTR = 1024 + 64;
+constexpr int E_TILE = 16 * E_ISTR;
+constexpr int E_STAGES = 2;
+
+#define PSA_LDS(T) __attribute__((address_space(3))) T*
+
+__global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
+  constexpr int D = 128, KK = D / 16, RS = 2;  // RS sets of 32 query rows per wave
+  __shared__ __align__(16) unsigned char smem[E_STAGES * E_TILE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int bh = blockIdx.y;
+  const int h = bh % p.Hq, b = bh / p.Hq;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int keep_m = 1 << p.keep_m_log2, keep_n = 1 << p.keep_n_log2;
+
+  // Q fragments: lane holds Q[row l32 of set rs][16*kk + 8*hh .. +8]
+  const int row0 = blockIdx.x * (4 * 32 * RS) + wave * (32 * RS);
+  bf16x8 qf[RS][KK];
+  {
+    const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * keep_m : nullptr;
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs) {
+      const int src = sampled_src(row0 + rs * 32 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
+      const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) qf[rs][kk] = *(const bf16x8*)(qp + kk * 16);
+    }
+  }
+
+  const char* kb = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  const uint32_t kstrb = (uint32_t)p.k_sl * 2u;
+  const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * keep_n : nullptr;
+  const int Ns = p.Ns, Lk = p.Lk, bn = p.bn, kn_log2 = p.keep_n_log2;
+
+  // fetch: wave w copies the 16-row group w of a tile; lane (q = lane/16, pos = lane%16) of block n writes
+  // row q of that block at position pos, i.e. tile slot 16w + 4q + n, chunk pos ^ q
+  const int fq = lane >> 4;
+  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
+  const int slot0 = wave * 16 + fq * 4;  // first of this lane's 4 consecutive tile slots (inside one key group)
+  int my_off[4];
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    const int e = (slot0 + n) & (keep_n - 1);
+    my_off[n] = ok ? ok[e] : e;
+  }
+  auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
+    const int r0 = t * TK + slot0;
+    const bool inside = (t + 1) * TK <= Ns && ((((t + 1) * TK - 1) >> kn_log2) + 1) * bn <= Lk;  // uniform
+    const int grp_row = (r0 >> kn_log2) * bn;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      int src = grp_row + my_off[n];
+      if (!inside) {
+        // padding keys replicate the last sampled key; rows past the sequence end clamp to its last row
+        int r = r0 + n;
+        if (r >= Ns) {
+          r = Ns - 1;
+          const int e = r & (keep_n - 1);
+          src = (r >> kn_log2) * bn + (ok ? ok[e] : e);
+        }
+        src = src < Lk ? src : Lk - 1;
+      }
+      __builtin_amdgcn_global_load_lds(kb + ((uint32_t)src * kstrb + f_chunk),
+                                       (PSA_LDS(void))(smem + stage * E_TILE + (wave * 4 + n) * E_ISTR), 16, 0, 0);
+    }
+  };
+  // K operand of k-step kk: tile slot l32 (+32) = block 4*(l32>>4) + (l32&3), row (l32>>2)&3, chunk 2kk + hh
+  // -> k_off[kk & 1] + 64 * (kk >> 1)   (+ 8 blocks for the second 32 keys)
+  uint32_t k_off[2];
+  {
+    const int q = (l32 >> 2) & 3;
+    const int base = (4 * (l32 >> 4) + (l32 & 3)) * E_ISTR + q * 256;
+    k_off[0] = (uint32_t)(base + ((hh ^ q) * 16));
+    k_off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
+  }
+
+  const int T = p.Ns_pad / TK;
+  const int gpc_log2 = 5 - p.keep_n_log2;  // key groups per 32-key chunk (1, 2 or 4)
+  float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + row0 + l32;
+  const int64_t rts = p.Ms_pad;
+  float m_run[RS];
+#pragma unroll
+  for (int rs = 0; rs < RS; ++rs) m_run[rs] = -INFINITY;
+  const float qk_scale = p.qk_scale;
+
+  // group maxima of the previous tile, written one tile late so that the stores' latency hides behind the MFMAs:
+  // per (row set, 32-key chunk) a lane owns at most 2 values (it stores for key group jbase + 2*i + hh, or for
+  // jbase when there is one group per chunk)
+  float pend[RS][2][2];
+  auto flush = [&](int tp) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int jbase = (tp * 2 + c) << gpc_log2;
+        float* rto = rt + rs * 32;
+        if (gpc_log2 == 0) {
+          if (hh == 0) rto[(int64_t)jbase * rts] = pend[rs][c][0];
+        } else if (gpc_log2 == 1) {
+          rto[(int64_t)(jbase + hh) * rts] = pend[rs][c][0];
+        } else {
+          rto[(int64_t)(jbase + hh) * rts] = pend[rs][c][0];
+          rto[(int64_t)(jbase + 2 + hh) * rts] = pend[rs][c][1];
+        }
+      }
+  };
+
+  // this workgroup's share of the key tiles
+  const int ks = blockIdx.z;
+  const int t_begin = (int)((int64_t)T * ks / p.ksplit), t_end = (int)((int64_t)T * (ks + 1) / p.ksplit);
+  issue_tile(t_begin, t_begin & 1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  for (int t = t_begin; t < t_end; ++t) {
+    // invariant: stage t&1 holds tile t and every wave is done with the other stage
+    if (t + 1 < t_end) issue_tile(t + 1, (t + 1) & 1);
+    if (t > t_begin) flush(t - 1);
+
+    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + (t & 1) * E_TILE;
+    f32x16 s[RS][2];
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[rs][c][i] = 0.f;
+    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 8 * E_ISTR);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      bf16x8 n0 = a0, n1 = a1;
+      if (kk + 1 < KK) {
+        n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
+        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + 8 * E_ISTR);
+      }
+#pragma unroll
+      for (int rs = 0; rs < RS; ++rs) {
+        s[rs][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[rs][kk], s[rs][0], 0, 0, 0);
+        s[rs][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[rs][kk], s[rs][1], 0, 0, 0);
+      }
+      a0 = n0;
+      a1 = n1;
+    }
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        // register i holds key (i/4)*8 + hh*4 + i%4 of this chunk: 8-key octets are registers 4o..4o+3
+        const f32x16& sc = s[rs][c];
+        if (gpc_log2 == 0) {
+          float v = sc[0];
+#pragma unroll
+          for (int i = 1; i < 15; i += 2) v = max3f(v, sc[i], sc[i + 1]);
+          v = half_wave_max(fmaxf(v, sc[15])) * qk_scale;
+          m_run[rs] = fmaxf(m_run[rs], v);
+          pend[rs][c][0] = v;
+        } else if (gpc_log2 == 1) {
+          float v0 = max3f(max3f(sc[0], sc[1], sc[2]), max3f(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
+          float v1 = max3f(max3f(sc[8], sc[9], sc[10]), max3f(sc[11], sc[12], sc[13]), fmaxf(sc[14], sc[15]));
+          v0 = half_wave_max(v0) * qk_scale;
+          v1 = half_wave_max(v1) * qk_scale;
+          m_run[rs] = max3f(m_run[rs], v0, v1);
+          pend[rs][c][0] = hh ? v1 : v0;
+        } else {
+          float v[4];
+#pragma unroll
+          for (int o = 0; o < 4; ++o) {
+            v[o] = half_wave_max(fmaxf(max3f(sc[4 * o], sc[4 * o + 1], sc[4 * o + 2]), sc[4 * o + 3])) * qk_scale;
+            m_run[rs] = fmaxf(m_run[rs], v[o]);
+          }
+          pend[rs][c][0] = hh ? v[1] : v[0];
+          pend[rs][c][1] = hh ? v[3] : v[2];
+        }
+      }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the copies of tile t+1 (and the stores of tile t-1) were issued a tile ago
+    __syncthreads();
+  }
+  if (t_end > t_begin) flush(t_end - 1);
+  if (hh == 0) {
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs) p.mrow[((int64_t)bh * p.ksplit + ks) * p.Ms_pad + row0 + rs * 32 + l32] = m_run[rs];
+  }
 }
 
 // one workgroup per (b, h, query group): Po[i, :] from R^T and m.
@@ -194,7 +388,8 @@ __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
   const int row = lane & (keep_m - 1), sub = lane >> p.keep_m_log2;
   const int per_iter = 64 >> p.keep_m_log2;  // key groups per wave iteration
   const int r0 = i * keep_m;
-  const float m = p.mrow[(int64_t)bh * p.Ms_pad + r0 + row];
+  float m = -INFINITY;
+  for (int ks = 0; ks < p.ksplit; ++ks) m = fmaxf(m, p.mrow[((int64_t)bh * p.ksplit + ks) * p.Ms_pad + r0 + row]);
   const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0 + row;
   for (int j0 = wave * per_iter; j0 < p.n_d; j0 += 4 * per_iter) {
     const int j = j0 + sub;
@@ -216,11 +411,25 @@ __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
 }
 
 template <int D>
-int launch_est(const EstParams& p, int B, hipStream_t stream) {
+int launch_est(EstParams& p, int B, hipStream_t stream) {
   constexpr int NW = 4;
   const int rows_needed = p.out_rows << p.keep_m_log2;
   dim3 grid((unsigned)((rows_needed + NW * 32 - 1) / (NW * 32)), (unsigned)(B * p.Hq));
-  hipLaunchKernelGGL((psa_est_gemm_kernel<D, NW>), grid, dim3(NW * 64), 0, stream, p);
+  p.ksplit = 1;
+  if (D == 128) {
+    // 256-row workgroups: cut the key range until about 3 workgroups per CU exist (the kernel's occupancy),
+    // keeping at least 8 key tiles per share
+    const int64_t wgs = (int64_t)((rows_needed + 255) / 256) * B * p.Hq;
+    const int tiles = p.Ns_pad / TK;
+    while (p.ksplit < EST_MAX_KSPLIT && wgs * p.ksplit < 3 * 256 && tiles / (p.ksplit * 2) >= 8) p.ksplit *= 2;
+  }
+  if (D == 128) {
+    grid.x = (unsigned)((rows_needed + 255) / 256);
+    grid.z = (unsigned)p.ksplit;
+    hipLaunchKernelGGL(psa_est_gemm128_kernel, grid, dim3(256), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((psa_est_gemm_kernel<D, NW>), grid, dim3(NW * 64), 0, stream, p);
+  }
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
   hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
@@ -235,8 +444,8 @@ EstGeom est_geom(int Lq, int Lk, int block_m, int block_n, int keep_m, int keep_
   const int Mq = (Lq + block_m - 1) / block_m, Nk = (Lk + block_n - 1) / block_n;
   g.Ms = Mq * keep_m;
   g.Ns = Nk * keep_n;
-  // the GEMM kernel works on 128 query rows per workgroup; the reference pads to 64
-  g.Ms_pad = (g.Ms + 127) / 128 * 128;
+  // the contraction kernels work on 128 or 256 query rows per workgroup; the reference pads to 64
+  g.Ms_pad = (g.Ms + 255) / 256 * 256;
   g.Ns_pad = (g.Ns + 63) / 64 * 64;
   g.m_d = ((g.Ms + 63) / 64 * 64) / keep_m;
   g.n_d = g.Ns_pad / keep_n;
@@ -248,7 +457,7 @@ EstGeom est_geom(int Lq, int Lk, int block_m, int block_n, int keep_m, int keep_
 extern "C" int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, int block_m, int block_n, int keep_m, int keep_n) {
   if (B <= 0 || Hq <= 0 || Lq <= 0 || Lk <= 0 || block_m <= 0 || block_n <= 0 || keep_m <= 0 || keep_n <= 0) return 0;
   const EstGeom g = est_geom(Lq, Lk, block_m, block_n, keep_m, keep_n);
-  return (int64_t)B * Hq * ((int64_t)g.n_d + 1) * g.Ms_pad * (int64_t)sizeof(float);
+  return (int64_t)B * Hq * ((int64_t)g.n_d + EST_MAX_KSPLIT) * g.Ms_pad * (int64_t)sizeof(float);
 }
 
 extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,

@@ -47,7 +47,7 @@ struct FwdParams {
   int64_t npad;
   float scale_log2;
   int causal;
-  int total_wg, wg_chunk;
+  int total_wg, wg_chunk, wg_groups;  // rows are dealt in wg_groups groups of wg_chunk; group g runs on XCD g % 8
   int max_tiles;
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
 };
@@ -126,7 +126,8 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
   // XCD-aware decode: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous range of (b, h, q-block) so that one XCD's L2 sees few heads at a time.
   const int bid = blockIdx.x;
-  int logical = (bid & 7) * p.wg_chunk + (bid >> 3);
+  // workgroup ids go round-robin over the 8 XCDs; slot s of XCD x works on row (s % chunk) of group 8*(s / chunk) + x
+  int logical = (((bid >> 3) / p.wg_chunk) * 8 + (bid & 7)) * p.wg_chunk + (bid >> 3) % p.wg_chunk;
   if (p.order != nullptr) logical = p.order[logical];
   if (logical < 0 || logical >= p.total_wg) return;
   const int I = logical % p.Mq;
@@ -502,7 +503,6 @@ constexpr int F_TILE = 16 * F_ISTR;   // bytes of one K or V tile (D = 128)
 
 #define PSA_LDS(T) __attribute__((address_space(3))) T*
 
-__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
 #define TILE_SYNC()                         \
   do {                                      \
@@ -533,7 +533,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
 
   const int bid = blockIdx.x;
-  int logical = (bid & 7) * p.wg_chunk + (bid >> 3);
+  // workgroup ids go round-robin over the 8 XCDs; slot s of XCD x works on row (s % chunk) of group 8*(s / chunk) + x
+  int logical = (((bid >> 3) / p.wg_chunk) * 8 + (bid & 7)) * p.wg_chunk + (bid >> 3) % p.wg_chunk;
   if (p.order != nullptr) logical = p.order[logical];
   if (logical < 0 || logical >= p.total_wg) return;
   const int I = logical % p.Mq;
@@ -690,10 +691,10 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     float mx0 = s_cur[0][0], mx1 = s_cur[1][0];
 #pragma unroll
     for (int i = 1; i < 15; i += 2) {
-      mx0 = max3(mx0, s_cur[0][i], s_cur[0][i + 1]);
-      mx1 = max3(mx1, s_cur[1][i], s_cur[1][i + 1]);
+      mx0 = max3f(mx0, s_cur[0][i], s_cur[0][i + 1]);
+      mx1 = max3f(mx1, s_cur[1][i], s_cur[1][i + 1]);
     }
-    float mx = max3(mx0, s_cur[0][15], fmaxf(mx1, s_cur[1][15]));
+    float mx = max3f(mx0, s_cur[0][15], fmaxf(mx1, s_cur[1][15]));
     mx = half_wave_max(mx);
     const float bias = (float)lv;
     const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
@@ -851,6 +852,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
 // to the 8 XCDs and each XCD runs its ids in order, so sorting every XCD's share by decreasing tile count
 // shortens the tail of the launch.  The order only changes WHEN a row is computed, never its result.
 constexpr int COST_BINS = 2048;
+constexpr int FWD_MAX_PHASES = 64;
+constexpr int64_t FWD_PHASE_BYTES = 128ll << 20;  // K/V (+ pooled levels) in use at one time
 
 __global__ __launch_bounds__(256) void psa_fwd_cost_kernel(const void* map, int map_elem, int total, int Mq, int Nk, int bn_log2,
                                                          int bm, int causal, int32_t* cost) {
@@ -877,7 +880,7 @@ __global__ __launch_bounds__(256) void psa_fwd_cost_kernel(const void* map, int 
   }
 }
 
-// one workgroup per XCD share: counting sort by decreasing cost
+// one workgroup per group of rows: counting sort by decreasing cost
 __global__ __launch_bounds__(256) void psa_fwd_sort_kernel(const int32_t* cost, int total, int chunk, int32_t* order) {
   __shared__ int hist[COST_BINS];
   const int x = blockIdx.x, tid = threadIdx.x;
@@ -887,12 +890,28 @@ __global__ __launch_bounds__(256) void psa_fwd_sort_kernel(const int32_t* cost, 
   for (int i = tid; i < chunk; i += 256)
     if (r0 + i < total) atomicAdd(&hist[cost[r0 + i]], 1);
   __syncthreads();
-  if (tid == 0) {  // start offset of every bin, highest cost first
-    int run = 0;
-    for (int b = COST_BINS - 1; b >= 0; --b) {
-      const int c = hist[b];
-      hist[b] = run;
-      run += c;
+  {  // start offset of every bin, highest cost first: thread i owns the 8 bins COST_BINS-1-8i .. COST_BINS-8-8i
+    __shared__ int part[256];
+    constexpr int PER = COST_BINS / 256;
+    int c[PER], sum = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      c[j] = hist[COST_BINS - 1 - (tid * PER + j)];
+      sum += c[j];
+    }
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the threads
+      const int add = tid >= d ? part[tid - d] : 0;
+      __syncthreads();
+      part[tid] += add;
+      __syncthreads();
+    }
+    int run = part[tid] - sum;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      hist[COST_BINS - 1 - (tid * PER + j)] = run;
+      run += c[j];
     }
   }
   __syncthreads();
@@ -913,7 +932,7 @@ int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
     if (hipFuncSetAttribute((const void*)psa_fwd_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
       return PSA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((psa_fwd_kernel<D, NW>), dim3((unsigned)(p.wg_chunk * 8)), dim3(NW * 64), shmem, stream, p);
+  hipLaunchKernelGGL((psa_fwd_kernel<D, NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
   return PSA_OK;
 }
 
@@ -923,7 +942,7 @@ int launch_fwd_d128(const FwdParams& p, int Nk, hipStream_t stream) {
   if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
   if (hipFuncSetAttribute((const void*)psa_fwd_d128_kernel<NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
     return PSA_ERR_LAUNCH;
-  hipLaunchKernelGGL((psa_fwd_d128_kernel<NW>), dim3((unsigned)(p.wg_chunk * 8)), dim3(NW * 64), shmem, stream, p);
+  hipLaunchKernelGGL((psa_fwd_d128_kernel<NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
   return PSA_OK;
 }
 
@@ -932,7 +951,7 @@ int launch_fwd_d128(const FwdParams& p, int Nk, hipStream_t stream) {
 extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
   if (B <= 0 || Hq <= 0 || L <= 0 || block_m <= 0) return 0;
   const int64_t total = (int64_t)B * Hq * ((L + block_m - 1) / block_m);
-  return 2 * 8 * ((total + 7) / 8) * (int64_t)sizeof(int32_t);
+  return 2 * (total + 8 * FWD_MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
 }
 
 extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
@@ -971,18 +990,28 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.scale_log2 = sm_scale * 1.4426950408889634f;
   p.causal = causal ? 1 : 0;
   p.total_wg = (int)total;
-  p.wg_chunk = (int)((total + 7) / 8);
+  // Groups of rows run one after the other on each XCD.  With several phases (8 groups each) the K/V of only a
+  // few heads is in use at a time, so that the part of it that misses L2 can stay in the last-level cache.
+  int phases = 1;
+  {
+    const double kv_bytes = 2.0 * B * Hkv * ((double)Nk * block_n) * D * 2.0 * (map != nullptr ? 1.875 : 1.0);
+    phases = (int)(kv_bytes / (double)FWD_PHASE_BYTES) + 1;
+    const int max_phases = B * Hkv < FWD_MAX_PHASES ? B * Hkv : FWD_MAX_PHASES;
+    phases = phases > max_phases ? max_phases : phases;
+  }
+  p.wg_groups = 8 * phases;
+  p.wg_chunk = (int)((total + p.wg_groups - 1) / p.wg_groups);
   // worst case: every kv-block at level 1, plus one partly filled tile per pooled level
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
   p.order = nullptr;
   if (workspace != nullptr && map != nullptr && total > 8 * 32) {
     PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
     int32_t* order = (int32_t*)workspace;
-    int32_t* cost = order + (int64_t)p.wg_chunk * 8;
+    int32_t* cost = order + (int64_t)p.wg_chunk * p.wg_groups;
     hipLaunchKernelGGL(psa_fwd_cost_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes,
                        (int)total, Mq, Nk, p.bn_log2, block_m, p.causal, cost);
     if (int e = psa_check_launch("psa_fwd (row cost)")) return e;
-    hipLaunchKernelGGL(psa_fwd_sort_kernel, dim3(8), dim3(256), 0, (hipStream_t)stream, cost, (int)total, p.wg_chunk, order);
+    hipLaunchKernelGGL(psa_fwd_sort_kernel, dim3(p.wg_groups), dim3(256), 0, (hipStream_t)stream, cost, (int)total, p.wg_chunk, order);
     if (int e = psa_check_launch("psa_fwd (row order)")) return e;
     p.order = order;
   }
