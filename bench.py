@@ -34,6 +34,10 @@ WORKLOADS = {
 WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
 
 
+# psa_fwd_d128_kernel at workload c2: (1080692.5 * 2.000 + 98280.0) KiB per dispatch
+FWD_TRAFFIC_BYTES = {"c2": 2.314e9}
+
+
 def scaled_ratios(tau):
     return {lv: (lo * tau if lv else 0.8 * tau, hi * tau if lv else 1.0) for lv, (lo, hi) in WAN13.items()}
 
@@ -156,9 +160,12 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command (scaled by the
+        # readings of --copy-calib's 1 GiB kernel); measured for the default workload only
+        "traffic": FWD_TRAFFIC_BYTES.get(args.workload),
         "flops_per_launch": exec_flops,
         "avg_launch_ms": round(t_fwd_avg, 4),
+        "launch_includes": "the forward kernel and its two row-ordering launches (about 9 us together)",
     }
 
     # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------
