@@ -112,11 +112,9 @@ def main():
     state = {}
 
     def layer():
-        kp, vp = ops.pool_kv(k, v, bn)
-        s = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
-        mp = ops.level_map(s, ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
-        o = ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp))
-        state.update(kp=kp, vp=vp, s=s, mp=mp, o=o)
+        # estimate -> level map -> pooling -> forward
+        o, mp = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+        state.update(mp=mp, o=o)
         return o
 
     # ---- the timed region: W warm-up steps, then exactly K steps --------------------------
@@ -133,7 +131,9 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_step = e0.elapsed_time(e1) / args.steps
 
-    mp, kp, vp = state["mp"], state["kp"], state["vp"]
+    mp = state["mp"]
+    kp, vp = ops.pool_kv(k, v, bn)
+    state["s"] = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
     density = float(ops.density(mp)[-1])
     dense_flops = 4.0 * L * L * D * H * B
     exec_flops = dense_flops * density

@@ -116,6 +116,19 @@ class PSAAttention(nn.Module):
         return mask
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        config = self.config
+        needs_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
+        if not needs_grad:
+            # inference: the stages back to back with a dense int8 level map (same levels as the mask formats)
+            if self.sample_offsets is None:
+                B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
+                off_q = draw_sample_offsets(B, H, config.block_m, config.block_m // 4, q.device)
+                off_k = draw_sample_offsets(B, Hkv, config.block_n, config.block_n // 4, k.device)
+            else:
+                off_q, off_k = self.sample_offsets
+            cap = calc_k_similarity(k, config.block_n, config) if config.use_sim_mask else None
+            return ops.psa_layer_fwd(q, k, v, off_q, off_k, config.mask_ratios, config.mask_mode, config.block_m,
+                                     config.block_n, config.tile_n, level_cap=cap)
         mask = self.build_mask(q, k, v)
         return self.sparse_attention_fn(q, k, v, mask, None)
 

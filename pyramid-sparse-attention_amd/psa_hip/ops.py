@@ -312,6 +312,41 @@ def sparse_attention_fwd(
     return res
 
 
+# ----------------------------------------------------------------------------- whole layer, forward only
+def psa_layer_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    off_q: torch.Tensor,
+    off_k: torch.Tensor,
+    mask_ratios,
+    mode: str,
+    block_m: int,
+    block_n: int,
+    tile_n: int,
+    sm_scale: Optional[float] = None,
+    level_cap: Optional[torch.Tensor] = None,
+    return_map: bool = False,
+):
+    """estimate -> level map -> pooled K/V -> sparse attention, non-causal, no gradient: the four stages
+    on the current stream with a dense int8 level map in between (no index-list round trip).  Running the
+    pooling pass on a second stream beside the level-map kernel was measured and gains nothing: the
+    level-map launch already occupies every wave slot of the chip."""
+    _require_gpu(q, k, v)
+    qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
+    keep_m, keep_n = block_m // 4, block_n // 4
+    sm_scale = qb.shape[-1] ** -0.5 if sm_scale is None else float(sm_scale)
+    scores = estimate_sampled(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, sm_scale)
+    mp = level_map(scores, mask_ratios, 0, mode, blocksize=block_n, compute_tile=tile_n, map_dtype=torch.int8)
+    if level_cap is not None:
+        mp = map_min_cap(mp, level_cap)
+    kp, vp = pool_kv(kb, vb, block_n)
+    out = sparse_attention_fwd(qb, kb, vb, mp, block_m, block_n, sm_scale, pools=(kp, vp))
+    if out.dtype != q.dtype:
+        out = out.to(q.dtype)
+    return (out, mp) if return_map else out
+
+
 # ----------------------------------------------------------------------------- attention backward
 def sparse_attention_bwd(
     q: torch.Tensor,

@@ -154,3 +154,24 @@ def test_pyramid_sparse_attention_text_tokens_cogvideo_preset():
     q, k, v = smooth_qkv(2, 2, (4, 8, 16), 64, 13, text=226)  # text tokens are appended at the end by make_qkv
     out = mod(q.to(dev()), k.to(dev()), v.to(dev()), 0)
     assert out.shape == q.shape and torch.isfinite(out).all()
+
+
+def test_layer_function_equals_the_stages_in_sequence():
+    """psa_layer_fwd: map and output must be bit-identical to the stages called one after the other."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    dev = torch.device("cuda:0")
+    B, H, D, bm, bn, tn = 1, 3, 128, 128, 128, 32
+    q, k, v = make_qkv(B, H, H, (4, 16, 40), D, seed=7, device=dev)  # L = 2560
+    off_q = sample_offsets(B, H, bm, bm // 4, 17, device=dev)
+    off_k = sample_offsets(B, H, bn, bn // 4, 18, device=dev)
+    ratios = {1: (0.0, 0.3), 2: (0.3, 0.4), 4: (0.4, 0.5), 8: (0.5, 0.6), 0: (0.6, 1.0)}
+    s = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, bm // 4, bn // 4)
+    mp = ops.level_map(s, ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
+    ref = ops.sparse_attention_fwd(q, k, v, mp, bm, bn)
+    for _ in range(2):
+        out, m2 = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+        torch.cuda.synchronize()
+        assert torch.equal(m2, mp)
+        assert torch.equal(out, ref)
