@@ -98,7 +98,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_kernel(BwdParams p) {
   unsigned char* Kt = smem + 2 * SM::ROW_BYTES;
   u32x2* tdesc = (u32x2*)(smem + SM::TILE_BYTES);
   uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
-  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5], s_wcnt[4 * (NT / 64)];
 
   const int I = blockIdx.x % p.Mq;
   const int bh = blockIdx.x / p.Mq;
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_kernel(BwdParams p) {
     jmax = ce < jmax ? ce : jmax;
   }
   const int T = build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, bn_log2, L, causal != 0,
-                                       (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff);
+                                       (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
 
   // Q and dO fragments of this wave's 32 rows (B operands), per-row delta and lse
   const int q_idx = I * BM + wave * 32 + l32;

@@ -530,7 +530,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   // K buffers at 0 and F_TILE, V buffers at 2*F_TILE and 3*F_TILE
   u32x2* tdesc = (u32x2*)(smem + 4 * F_TILE);
   uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
-  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5], s_wcnt[4 * NW];
 
   const int bid = blockIdx.x;
   // workgroup ids go round-robin over the 8 XCDs; slot s of XCD x works on row (s % chunk) of group 8*(s / chunk) + x
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
   }
   const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2,
-                                                 P_L, P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff);
+                                                 P_L, P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
 
   const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
   const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);

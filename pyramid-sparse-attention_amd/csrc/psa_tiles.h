@@ -35,30 +35,59 @@ struct RowSchedule {
 
 // Builds ids[] (kv-block ids grouped by level, ascending inside a level) and tdesc[] for the map row
 // of (bh, q-block I).  Must be called by every thread of the workgroup; contains barriers.
-// s_cnt / s_ioff / s_toff are 4 / 4 / 5 ints of LDS scratch.
+// s_cnt / s_ioff / s_toff are 4 / 4 / 5 ints of LDS scratch; s_wcnt holds 4 ints per wave.
+// Every wave compacts one contiguous share of the row: counts first (one pass over the map row), then,
+// once the per-wave counts are known to all, the ids (second pass; the row is in cache by then).
 template <int NT>
 __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem, int64_t mrow, int Nk, int jmax, int bn_log2,
                                                   int L, bool causal, int64_t q_first_row, uint16_t* ids, u32x2* tdesc,
-                                                  int* s_cnt, int* s_ioff, int* s_toff) {
+                                                  int* s_cnt, int* s_ioff, int* s_toff, int* s_wcnt) {
+  constexpr int NW = NT / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (wave == 0) {
-    int cnt[4] = {0, 0, 0, 0};
-    if (map == nullptr) {
-      cnt[0] = jmax;
-      for (int j = lane; j < jmax; j += 64) ids[j] = (uint16_t)j;
-    } else {
-      for (int j0 = 0; j0 < jmax; j0 += 64) {
-        const int j = j0 + lane;
-        const int lvl = j < jmax ? load_map(map, mrow + j, map_elem) : 0;
+  // wave w owns columns [w * share, min(jmax, (w + 1) * share)), share a multiple of 64
+  const int share = ((jmax + 64 * NW - 1) / (64 * NW)) * 64;
+  const int j_lo = wave * share, j_hi = (wave + 1) * share < jmax ? (wave + 1) * share : jmax;
+  int cnt[4] = {0, 0, 0, 0};
+  if (map == nullptr) {
+    cnt[0] = j_hi > j_lo ? j_hi - j_lo : 0;
+  } else {
+    for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
+      const int j = j0 + lane;
+      const int lvl = j < j_hi ? load_map(map, mrow + j, map_elem) : 0;
 #pragma unroll
-        for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
+      for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) s_wcnt[wave * 4 + lv] = cnt[lv];
+  }
+  __syncthreads();
+  {
+    // offsets of this wave's share inside each level list; totals for the tile bookkeeping
+    int run[4], tot[4];
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) {
+      int before = 0, all = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const int c = s_wcnt[w * 4 + lv];
+        before += w < wave ? c : 0;
+        all += c;
       }
-      int run[4];
-      run[0] = 0; run[1] = cnt[0]; run[2] = cnt[0] + cnt[1]; run[3] = cnt[0] + cnt[1] + cnt[2];
+      run[lv] = before;
+      tot[lv] = all;
+    }
+    run[1] += tot[0];
+    run[2] += tot[0] + tot[1];
+    run[3] += tot[0] + tot[1] + tot[2];
+    if (map == nullptr) {
+      for (int j = j_lo + lane; j < j_hi; j += 64) ids[j] = (uint16_t)j;
+    } else {
       const uint64_t lt_mask = (1ull << lane) - 1ull;
-      for (int j0 = 0; j0 < jmax; j0 += 64) {
+      for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
         const int j = j0 + lane;
-        const int lvl = j < jmax ? load_map(map, mrow + j, map_elem) : 0;
+        const int lvl = j < j_hi ? load_map(map, mrow + j, map_elem) : 0;
 #pragma unroll
         for (int lv = 0; lv < 4; ++lv) {
           const uint64_t bal = __ballot(lvl == (1 << lv));
@@ -67,11 +96,11 @@ __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem,
         }
       }
     }
-    if (lane == 0) {
+    if (tid == 0) {
       int io = 0, to = 0;
 #pragma unroll
       for (int lv = 0; lv < 4; ++lv) {
-        const int c = lv == 0 ? cnt[0] : lv == 1 ? cnt[1] : lv == 2 ? cnt[2] : cnt[3];
+        const int c = tot[lv];
         const int sbs_log2 = bn_log2 - lv;
         s_cnt[lv] = c;
         s_ioff[lv] = io;
