@@ -14,6 +14,8 @@
 //                          <= 64 pooled keys in registers and streams the q-blocks that retain this block at
 //                          this level; dK_l, dV_l go to an fp32 workspace (every row written exactly once)
 //   psa_bwd_unpool_kernel  HBM-bound: sums the levels, spreads pooled gradients, folds the pad tail, -> bf16
+#include <type_traits>
+
 #include "psa_tiles.h"
 
 namespace {
@@ -385,9 +387,11 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int s
     int64_t row = key_row0 + (key_local < key_valid ? key_local : 0);
     if (key_valid == 0) row = 0;
     const bf16_t *kp_, *vp_;
-    if (lv == 0) {
-      kp_ = p.k + b * p.k_sb + hk * p.k_sh + row * p.k_sl;
-      vp_ = p.v + b * p.v_sb + hk * p.v_sh + row * p.v_sl;
+    if (lv == 0 || p.kp == nullptr) {
+      // without a level map there are no pooled buffers: the workgroups of the pooled levels have an empty
+      // q-block list and only write zeros, whatever they load here
+      kp_ = p.k + b * p.k_sb + hk * p.k_sh + (lv == 0 ? row : 0) * p.k_sl;
+      vp_ = p.v + b * p.v_sb + hk * p.v_sh + (lv == 0 ? row : 0) * p.v_sl;
     } else {
       const int64_t off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + row) * D;
       kp_ = p.kp + off;
@@ -561,6 +565,323 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int s
 }
 
 // ------------------------------------------------------------------------------------------------------
+// dK/dV column walk, head dim 128: Q and dO rows are copied from global memory straight into LDS (double
+// buffered, one barrier per step of 64 query rows) in the padded + swizzled row-major tile layout of the forward
+// kernel; the row operands (S = Q K^T, dP = dO V^T) are 128-bit LDS reads and the transposed operands
+// (dV^T += dO^T P, dK^T += Q^T dS) come from the same tiles through the transposing LDS load.
+// ------------------------------------------------------------------------------------------------------
+constexpr int B_ISTR = 1024 + 64;    // bytes between the 4-row blocks of a tile
+constexpr int B_TILE = 16 * B_ISTR;  // 64 rows x 256 bytes, padded
+
+#define PSA_LDS(T) __attribute__((address_space(3))) T*
+
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, int slots_per_block) {
+  constexpr int D = 128, KK = D / 16, DB = D / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  // stage s: Q tile at 2*s*B_TILE, dO tile at (2*s + 1)*B_TILE
+  float* s_lse = (float*)(smem + 4 * B_TILE);  // [2 stages][64]
+  float* s_del = s_lse + 128;                  // [2 stages][64]
+  uint32_t* qlist = (uint32_t*)(s_del + 128);  // [n_rep * Mq]  (head in group << 16 | q-block)
+  __shared__ int s_nq;
+
+  const int slot = blockIdx.x % slots_per_block;
+  const int J = blockIdx.x / slots_per_block;
+  const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  const int n_rep = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal, bm = p.bm, Mq = p.Mq;
+
+  int lv, part;
+  decode_slot(slot, bn_log2, lv, part);
+  const int sbs = 1 << (bn_log2 - lv);            // pooled keys of this block at this level
+  const int nkeys = sbs < 64 ? sbs : 64;
+  const int64_t key_row0 = ((int64_t)J << (bn_log2 - lv)) + part * 64;  // first pooled row of this workgroup
+  int key_valid = nkeys;                          // level 0: rows past L do not exist
+  if (lv == 0) {
+    const int64_t rem = (int64_t)L - key_row0;
+    key_valid = rem < nkeys ? (rem > 0 ? (int)rem : 0) : nkeys;
+  }
+  // waves = 2 key halves x 2 query halves.  With at most 32 keys only one key half works: alternate which
+  // pair of waves that is from workgroup to workgroup, so that all four SIMDs of a CU get work.
+  const int flip = nkeys <= 32 ? (int)((blockIdx.x + blockIdx.y) & 1) : 0;
+  const int kh = (wave & 1) ^ flip, qh = wave >> 1;
+  const bool wave_active = key_valid > kh * 32;
+
+  // ---- list of (head in group, q-block) that retain block J at this level -------------------------
+  if (wave == 0) {
+    int n = 0;
+    const int total = n_rep * Mq;
+    for (int e0 = 0; e0 < total; e0 += 64) {
+      const int e = e0 + lane;
+      bool on = false;
+      if (e < total) {
+        const int hl = e / Mq, I = e % Mq;
+        const int h = hk * n_rep + hl;
+        int level = p.map ? load_map(p.map, (((int64_t)b * p.Hq + h) * Mq + I) * p.Nk + J, p.map_elem) : 1;
+        if (causal) {
+          const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
+          if (J >= ce) level = 0;
+        }
+        on = level == (1 << lv);
+      }
+      const uint64_t bal = __ballot(on);
+      if (on) qlist[n + __popcll(bal & ((1ull << lane) - 1ull))] = ((uint32_t)(e / Mq) << 16) | (uint32_t)(e % Mq);
+      n += __popcll(bal);
+    }
+    if (lane == 0) s_nq = n;
+  }
+
+  // ---- this wave's 32 keys: K and V fragments (B operands) --------------------------------------------
+  const int key_local = kh * 32 + l32;
+  bf16x8 kf[KK], vf[KK];
+  {
+    int64_t row = key_row0 + (key_local < key_valid ? key_local : 0);
+    if (key_valid == 0) row = 0;
+    const bf16_t *kp_, *vp_;
+    if (lv == 0 || p.kp == nullptr) {
+      // without a level map there are no pooled buffers: the workgroups of the pooled levels have an empty
+      // q-block list and only write zeros, whatever they load here
+      kp_ = p.k + b * p.k_sb + hk * p.k_sh + (lv == 0 ? row : 0) * p.k_sl;
+      vp_ = p.v + b * p.v_sb + hk * p.v_sh + (lv == 0 ? row : 0) * p.v_sl;
+    } else {
+      const int64_t off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + row) * D;
+      kp_ = p.kp + off;
+      vp_ = p.vp + off;
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      kf[kk] = *(const bf16x8*)(kp_ + kk * 16 + hh * 8);
+      vf[kk] = *(const bf16x8*)(vp_ + kk * 16 + hh * 8);
+    }
+  }
+  const bool key_ok = key_local < key_valid;
+  const int key_up = (int)(((key_row0 + key_local + 1) << lv) - 1);  // last token the pooled key covers (< npad)
+  __syncthreads();
+  const int nq = s_nq;
+
+  // ---- lane-invariant LDS addressing (tile layout: see the forward kernel) ---------------------------
+  // copy: wave w fills the 16-row group w of both tiles; lane (fq = lane/16, pos = lane%16) of block n writes
+  // row fq of that block, i.e. tile row 16w + 4fq + n, chunk pos ^ fq
+  const int fq = lane >> 4;
+  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
+  const int f_row = wave * 16 + fq * 4;
+  // row operand of k-step kk for tile row qh*32 + l32: r_off[kk & 1] + 64 * (kk >> 1)
+  uint32_t r_off[2];
+  {
+    const int rw = qh * 32 + l32, q4 = (rw >> 2) & 3;
+    const int base = (4 * (rw >> 4) + (rw & 3)) * B_ISTR + q4 * 256;
+    r_off[0] = (uint32_t)(base + ((hh ^ q4) * 16));
+    r_off[1] = (uint32_t)(base + (((2 + hh) ^ q4) * 16));
+  }
+  // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
+  uint32_t t_off[2];
+  {
+    const int i16 = lane & 15, bl = lane >> 4;
+    const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const int qq = 2 * s2 + (bl >> 1);
+      t_off[s2] = (uint32_t)(n * B_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
+    }
+  }
+
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      dk[db][i] = 0.f;
+      dv[db][i] = 0.f;
+    }
+  const float scale_log2 = p.scale_log2;
+  const float bias = (float)lv;
+  const int spb = bm / 64;           // steps per q-block
+  const int n_steps = key_valid > 0 ? nq * spb : 0;
+  const uint32_t q_strb = (uint32_t)p.q_sl * 2u, do_strb = (uint32_t)p.do_sl * 2u;
+
+  // step i -> (head, q-block, first query row)
+  auto step_of = [&](int i, int& h, int& I, int& q0) __attribute__((always_inline)) {
+    const uint32_t ent = qlist[i / spb];
+    h = hk * n_rep + (int)(ent >> 16);
+    I = (int)(ent & 0xffff);
+    q0 = I * bm + (i % spb) * 64;
+  };
+  // rows of step i -> stage; the per-row lse / delta values come back in registers and are put into LDS later
+  float lse_next = 0.f, del_next = 0.f;
+  auto issue_step = [&](int i, int stage) __attribute__((always_inline)) {
+    int h, I, q0;
+    step_of(i, h, I, q0);
+    h = __builtin_amdgcn_readfirstlane(h);
+    q0 = __builtin_amdgcn_readfirstlane(q0);
+    if (tid < 64) {
+      const int row = q0 + tid;
+      const int64_t bh = (int64_t)b * p.Hq + h;
+      // rows past L: p is forced to 0 through lse = +inf
+      lse_next = row < L ? p.lse2[bh * L + row] : INFINITY;
+      del_next = row < L ? p.delta[bh * L + row] : 0.f;
+    }
+    const char* qb = (const char*)(p.q + b * p.q_sb + h * p.q_sh);
+    const char* ob = (const char*)(p.dout + b * p.do_sb + h * p.do_sh);
+    const int r0 = q0 + f_row;
+    if (q0 + 64 <= L) {
+      const uint32_t qo = (uint32_t)r0 * q_strb + f_chunk, oo = (uint32_t)r0 * do_strb + f_chunk;
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        __builtin_amdgcn_global_load_lds(qb + (uint64_t)(n * q_strb) + qo,
+                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(ob + (uint64_t)(n * do_strb) + oo,
+                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        int row = r0 + n;
+        row = row < L ? row : L - 1;
+        row = row > 0 ? row : 0;
+        __builtin_amdgcn_global_load_lds(qb + ((uint32_t)row * q_strb + f_chunk),
+                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(ob + ((uint32_t)row * do_strb + f_chunk),
+                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+      }
+    }
+  };
+  auto publish_rows = [&](int stage) __attribute__((always_inline)) {
+    if (tid < 64) {
+      s_lse[stage * 64 + tid] = lse_next;
+      s_del[stage * 64 + tid] = del_next;
+    }
+  };
+
+  PSA_LDS(const float) rows_base = (PSA_LDS(const float))(smem + 4 * B_TILE) + (qh * 32 + hh * 4);
+  auto compute_step = [&](int i, auto stage_c) __attribute__((always_inline)) {
+    constexpr int ST = decltype(stage_c)::value;
+    int h, I, q0;
+    step_of(i, h, I, q0);
+    I = __builtin_amdgcn_readfirstlane(I);
+    q0 = __builtin_amdgcn_readfirstlane(q0);
+    const bool diag = causal && ((((int64_t)J + 1) << bn_log2) - 1 > (int64_t)I * bm);
+    PSA_LDS(unsigned char) Qs = (PSA_LDS(unsigned char))(smem) + 2 * ST * B_TILE;
+    PSA_LDS(unsigned char) Os = (PSA_LDS(unsigned char))(smem) + (2 * ST + 1) * B_TILE;
+    // S = Q K^T and dP = dO V^T for this wave's (32 q) x (32 keys): lane = key column, registers = q rows
+    f32x16 s, dp;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      s[j] = 0.f;
+      dp[j] = 0.f;
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const bf16x8 qa = *(PSA_LDS(const bf16x8))(Qs + r_off[kk & 1] + (kk >> 1) * 64);
+      const bf16x8 oa = *(PSA_LDS(const bf16x8))(Os + r_off[kk & 1] + (kk >> 1) * 64);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[kk], dp, 0, 0, 0);
+    }
+    uint32_t pk[8], dsk[8];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int qq = qh * 32 + g * 8 + hh * 4;
+      // one lane base + immediates (stage, group, lse / delta array)
+      const f32x4 l4 = *(PSA_LDS(const f32x4))(rows_base + ST * 64 + g * 8);
+      const f32x4 d4 = *(PSA_LDS(const f32x4))(rows_base + 128 + ST * 64 + g * 8);
+      float pv[4], dsv[4];
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        float pe = fast_exp2(__builtin_fmaf(s[g * 4 + e2], scale_log2, bias - l4[e2]));
+        bool ok = key_ok;
+        if (diag) ok = ok && (key_up <= q0 + qq + e2);
+        pe = ok ? pe : 0.f;
+        pv[e2] = pe;
+        dsv[e2] = pe * (dp[g * 4 + e2] - d4[e2]);
+      }
+      pk[g * 2] = pack_bf16x2(pv[0], pv[1]);
+      pk[g * 2 + 1] = pack_bf16x2(pv[2], pv[3]);
+      dsk[g * 2] = pack_bf16x2(dsv[0], dsv[1]);
+      dsk[g * 2 + 1] = pack_bf16x2(dsv[2], dsv[3]);
+    }
+    // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over this wave's 32 query rows, 16 at a time)
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
+      u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
+      const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
+      const int grp = (2 * qh + g) * (4 * B_ISTR);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const u32x2 olo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[0] + db * 64 + grp)));
+        const u32x2 ohi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[1] + db * 64 + grp)));
+        u32x4 oa = {olo[0], olo[1], ohi[0], ohi[1]};
+        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, oa), pfrag, dv[db], 0, 0, 0);
+        const u32x2 qlo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Qs + t_off[0] + db * 64 + grp)));
+        const u32x2 qhi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Qs + t_off[1] + db * 64 + grp)));
+        u32x4 qa2 = {qlo[0], qlo[1], qhi[0], qhi[1]};
+        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qa2), sfrag, dk[db], 0, 0, 0);
+      }
+    }
+  };
+
+  if (n_steps > 0) {
+    issue_step(0, 0);
+    publish_rows(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the rows have landed
+    __syncthreads();
+    const std::integral_constant<int, 0> S0;
+    const std::integral_constant<int, 1> S1;
+    for (int i = 0; i < n_steps; i += 2) {
+      // invariant: stage i&1 holds step i, the other stage is free
+      if (i + 1 < n_steps) issue_step(i + 1, 1);
+      if (wave_active) compute_step(i, S0);
+      if (i + 1 < n_steps) publish_rows(1);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      if (i + 1 < n_steps) {
+        if (i + 2 < n_steps) issue_step(i + 2, 0);
+        if (wave_active) compute_step(i + 1, S1);
+        if (i + 2 < n_steps) publish_rows(0);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+      }
+    }
+  }
+
+  // ---- combine the two query halves and write this workgroup's rows of the level buffers ------------
+  __syncthreads();
+  float* red = (float*)smem;  // [2 key halves][2 tensors][DB*16][64 lanes]
+  if (qh == 1) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane] = dk[db][i];
+        red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane] = dv[db][i];
+      }
+  }
+  __syncthreads();
+  if (qh == 0 && key_local < nkeys) {
+    const int64_t lvl_off = pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad);
+    // level buffers: level 0 first ([BHkv, npad, D]), then levels 1..3 like the pooled K/V buffers
+    const int64_t base_rows = lv == 0 ? bhk * p.npad : (int64_t)p.B * p.Hkv * p.npad + lvl_off;
+    float* wk = p.wk + (base_rows + key_row0 + key_local) * D;
+    float* wv = p.wv + (base_rows + key_row0 + key_local) * D;
+    const float scale = p.scale;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 a, c2;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+          const int i = g * 4 + e2;
+          a[e2] = (dk[db][i] + red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane]) * scale;
+          c2[e2] = dv[db][i] + red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane];
+        }
+        *(f32x4*)(wk + db * 32 + g * 8 + hh * 4) = a;
+        *(f32x4*)(wv + db * 32 + g * 8 + hh * 4) = c2;
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------
 // un-pool: levels -> dK, dV (bf16)
 // ------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void psa_bwd_unpool_kernel(BwdParams p, int D) {
@@ -719,7 +1040,8 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       hipLaunchKernelGGL(kern, grid, dim3(256), shmem, st, p, spb);
       return PSA_OK;
     };
-    int rc = D == 128 ? launch(psa_bwd_dkdv_kernel<128>, KvSmem<128>::STAGE_BYTES) : launch(psa_bwd_dkdv_kernel<64>, KvSmem<64>::STAGE_BYTES);
+    int rc = D == 128 ? launch(psa_bwd_dkdv128_kernel, (size_t)4 * B_TILE + 128 * sizeof(float))
+                      : launch(psa_bwd_dkdv_kernel<64>, KvSmem<64>::STAGE_BYTES);
     PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
     rc = psa_check_launch("psa_bwd (dK/dV)");
     if (rc != PSA_OK) return rc;
