@@ -290,6 +290,202 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_kernel(BwdParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------------
+// dQ row walk, head dim 128: the forward's data path.  K and V tiles are copied from global memory straight
+// into double-buffered LDS tiles (layout: psa_tiles.h), one barrier per tile; S^T = K Q^T and dP^T = V dO^T
+// read them row-wise (128-bit reads), dQ^T += K^T dS^T reads the K tile through the transposing LDS load.
+// ------------------------------------------------------------------------------------------------------
+template <int NW>
+__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) {
+  constexpr int D = 128, NT = NW * 64, BM = NW * 32, CH = D / 8, KK = D / 16, DB = D / 32;
+  constexpr int G16 = 4 / NW;
+  constexpr int OST = D * 2 + 16;
+  static_assert(BM * OST <= 4 * LT_TILE, "dQ staging must fit the tile buffers");
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  // K tiles at 0 and LT_TILE, V tiles at 2*LT_TILE and 3*LT_TILE
+  u32x2* tdesc = (u32x2*)(smem + 4 * LT_TILE);
+  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
+  __shared__ int s_cnt[4], s_ioff[4], s_toff[5], s_wcnt[4 * NW];
+
+  const int I = blockIdx.x % p.Mq;
+  const int bh = blockIdx.x / p.Mq;
+  const int h = bh % p.Hq, b = bh / p.Hq;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal;
+  const float scale_log2 = p.scale_log2;
+
+  int jmax = p.Nk;
+  if (causal) {
+    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << bn_log2) - 1) >> bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  // Q and dO fragments of this wave's 32 rows (B operands), per-row delta and lse
+  const int q_idx = I * BM + wave * 32 + l32;
+  const int qr = q_idx < L ? q_idx : L - 1;
+  bf16x8 qf[KK], dof[KK];
+  {
+    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+    const bf16_t* dp_ = p.dout + b * p.do_sb + h * p.do_sh + (int64_t)qr * p.do_sl + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qf[kk] = *(const bf16x8*)(qp + kk * 16);
+      dof[kk] = *(const bf16x8*)(dp_ + kk * 16);
+    }
+  }
+  const float delta = q_idx < L ? p.delta[(int64_t)bh * L + q_idx] : 0.f;
+  const float lse2 = q_idx < L ? p.lse2[(int64_t)bh * L + q_idx] : INFINITY;
+
+  const int T = build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, bn_log2, L, causal != 0,
+                                       (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
+
+  KvSource kvs;
+  kvs.k0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  kvs.v0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
+  kvs.kp = (const char*)p.kp; kvs.vp = (const char*)p.vp;
+  kvs.k_strb = (uint32_t)p.k_sl * 2u; kvs.v_strb = (uint32_t)p.v_sl * 2u;
+  kvs.BHkv = (int64_t)p.B * p.Hkv; kvs.bhk = (int64_t)b * p.Hkv + hk; kvs.npad = p.npad;
+  kvs.bn_log2 = bn_log2; kvs.L = L;
+  const uint32_t f_chunk = lt_fetch_chunk(lane);
+  uint32_t r_off[2], t_off[2];
+  lt_row_operand(l32, hh, r_off);  // tile rows l32 (+32): r_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
+  lt_tr_operand(lane, t_off);      // K^T: t_off[s] + 64 * db + 4 * LT_ISTR * (16-key group)
+
+  auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
+    TileSrc<G16> ts;
+    lt_tile_src<G16>(kvs, tdesc, ids, t, wave, lane, ts);
+    lt_issue_rows<G16>(smem + stage * LT_TILE, ts.kbase, ts.kstr, ts.lim, ts.src0, wave, f_chunk);
+    lt_issue_rows<G16>(smem + (2 + stage) * LT_TILE, ts.vbase, ts.vstr, ts.lim, ts.src0, wave, f_chunk);
+  };
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+
+  auto compute_tile = [&](int t, auto stage_c) __attribute__((always_inline)) {
+    constexpr int ST = decltype(stage_c)::value;
+    const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
+    const int lv = d & 3;
+    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + ST * LT_TILE;
+    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + ST) * LT_TILE;
+    f32x16 s[2], dp[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[c][i] = 0.f;
+        dp[c][i] = 0.f;
+      }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const bf16x8 ka = *(PSA_LDS(const bf16x8))(Ks + r_off[kk & 1] + (kk >> 1) * 64 + c * 8 * LT_ISTR);
+        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s[c], 0, 0, 0);
+        const bf16x8 va = *(PSA_LDS(const bf16x8))(Vs + r_off[kk & 1] + (kk >> 1) * 64 + c * 8 * LT_ISTR);
+        dp[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp[c], 0, 0, 0);
+      }
+    }
+    if (d & 4) {
+      // Partly empty tile and/or causal diagonal: valid slots are a prefix of the tile (nvalid); a pooled key of
+      // level lv is visible to query i iff src < (i + 1) >> lv.  Each run of 4 slots keeps its first `keep`.
+      const int nvalid = (int)((d >> 3) & 127);
+      const int qlim = (q_idx + 1) >> lv;
+      const uint32_t d1 = __builtin_amdgcn_readfirstlane(tdesc[t][1]);
+      const int cnt = (int)(d1 >> 16), lt = (int)(d >> 10), sbs_log2 = bn_log2 - lv;
+      const uint16_t* lids = ids + (d1 & 0xffff);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int r0 = c * 32 + g * 8 + hh * 4;
+          int keep = nvalid - r0;
+          if (causal) {
+            const int gpos = (lt << 6) + r0;
+            int bi = gpos >> sbs_log2;
+            bi = bi < cnt - 1 ? bi : cnt - 1;
+            const int src0 = ((int)lids[bi] << sbs_log2) + (gpos & ((1 << sbs_log2) - 1));
+            keep = keep < qlim - src0 ? keep : qlim - src0;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[c][g * 4 + e] = e < keep ? s[c][g * 4 + e] : -INFINITY;
+        }
+    }
+    const float nb = (float)lv - lse2;
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = fast_exp2(__builtin_fmaf(s[c][i], scale_log2, nb));
+        const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], scale_log2, nb));
+        pk[c][i >> 1] = pack_bf16x2(p0 * (dp[c][i] - delta), p1 * (dp[c][i + 1] - delta));
+      }
+    // dQ^T += K^T dS^T
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg) {
+      const int c = cg >> 1, g = cg & 1;
+      u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
+      const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[0] + db * 64 + cg * (4 * LT_ISTR))));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[1] + db * 64 + cg * (4 * LT_ISTR))));
+        u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+      }
+    }
+  };
+
+  if (T > 0) {
+    // the Q / dO fragments must have arrived before the first copy is issued (a pending ordinary load would make
+    // the compiler wait for all copies in flight inside the loop)
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    issue_tile(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    const std::integral_constant<int, 0> S0;
+    const std::integral_constant<int, 1> S1;
+    for (int t = 0; t < T; t += 2) {
+      // invariant: stage t&1 holds tile t, the other stage is free
+      if (t + 1 < T) issue_tile(t + 1, 1);
+      compute_tile(t, S0);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      if (t + 1 < T) {
+        if (t + 2 < T) issue_tile(t + 2, 0);
+        compute_tile(t + 1, S1);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+      }
+    }
+  }
+
+  __syncthreads();
+  unsigned char* Os = smem;
+  const float scale = p.scale;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * scale, acc[db][g * 4 + 1] * scale);
+      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * scale, acc[db][g * 4 + 3] * scale);
+      *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
+    }
+  __syncthreads();
+  bf16_t* ob = p.dq + b * p.dq_sb + h * p.dq_sh;
+  for (int u = tid; u < BM * CH; u += NT) {
+    const int rr = u / CH, ch = u % CH;
+    const int row = I * BM + rr;
+    if (row < L) *(u32x4*)(ob + (int64_t)row * p.dq_sl + ch * 8) = *(const u32x4*)(Os + rr * OST + ch * 16);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------
 // dK, dV: column walk
 // ------------------------------------------------------------------------------------------------------
 template <int D>
@@ -570,10 +766,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int s
 // kernel; the row operands (S = Q K^T, dP = dO V^T) are 128-bit LDS reads and the transposed operands
 // (dV^T += dO^T P, dK^T += Q^T dS) come from the same tiles through the transposing LDS load.
 // ------------------------------------------------------------------------------------------------------
-constexpr int B_ISTR = 1024 + 64;    // bytes between the 4-row blocks of a tile
-constexpr int B_TILE = 16 * B_ISTR;  // 64 rows x 256 bytes, padded
-
-#define PSA_LDS(T) __attribute__((address_space(3))) T*
+constexpr int B_ISTR = LT_ISTR;  // bytes between the 4-row blocks of a tile
+constexpr int B_TILE = LT_TILE;  // 64 rows x 256 bytes, padded
 
 __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, int slots_per_block) {
   constexpr int D = 128, KK = D / 16, DB = D / 32;
@@ -663,28 +857,11 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
   // ---- lane-invariant LDS addressing (tile layout: see the forward kernel) ---------------------------
   // copy: wave w fills the 16-row group w of both tiles; lane (fq = lane/16, pos = lane%16) of block n writes
   // row fq of that block, i.e. tile row 16w + 4fq + n, chunk pos ^ fq
-  const int fq = lane >> 4;
-  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
-  const int f_row = wave * 16 + fq * 4;
-  // row operand of k-step kk for tile row qh*32 + l32: r_off[kk & 1] + 64 * (kk >> 1)
-  uint32_t r_off[2];
-  {
-    const int rw = qh * 32 + l32, q4 = (rw >> 2) & 3;
-    const int base = (4 * (rw >> 4) + (rw & 3)) * B_ISTR + q4 * 256;
-    r_off[0] = (uint32_t)(base + ((hh ^ q4) * 16));
-    r_off[1] = (uint32_t)(base + (((2 + hh) ^ q4) * 16));
-  }
-  // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
-  uint32_t t_off[2];
-  {
-    const int i16 = lane & 15, bl = lane >> 4;
-    const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      const int qq = 2 * s2 + (bl >> 1);
-      t_off[s2] = (uint32_t)(n * B_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
-    }
-  }
+  const uint32_t f_chunk = lt_fetch_chunk(lane);
+  const int f_row = wave * 16 + lt_fetch_row(lane);
+  uint32_t r_off[2], t_off[2];
+  lt_row_operand(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
+  lt_tr_operand(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -1017,8 +1194,8 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       return PSA_OK;
     };
     int rc;
-    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq_kernel<128, 4>, DqSmem<128>::TILE_BYTES, 4);
-    else if (D == 128) rc = launch(psa_bwd_dq_kernel<128, 2>, DqSmem<128>::TILE_BYTES, 2);
+    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq128_kernel<4>, (size_t)4 * LT_TILE, 4);
+    else if (D == 128) rc = launch(psa_bwd_dq128_kernel<2>, (size_t)4 * LT_TILE, 2);
     else if (block_m == 128) rc = launch(psa_bwd_dq_kernel<64, 4>, DqSmem<64>::TILE_BYTES, 4);
     else rc = launch(psa_bwd_dq_kernel<64, 2>, DqSmem<64>::TILE_BYTES, 2);
     PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: sequence too long for the on-chip schedule (LDS)");

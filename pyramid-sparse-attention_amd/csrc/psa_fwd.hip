@@ -498,10 +498,8 @@ __global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams
 //  * ds_read_b64_tr_b16 hands every lane 4 keys of one channel from row-major V: exactly the A operand
 //    of O^T += V^T P^T, in the key order that the S^T accumulator layout gives P^T.
 //  * The tile loop is unrolled by two so that the LDS buffer offsets are immediates.
-constexpr int F_ISTR = 1024 + 64;     // bytes between the 4-row blocks of a tile
-constexpr int F_TILE = 16 * F_ISTR;   // bytes of one K or V tile (D = 128)
-
-#define PSA_LDS(T) __attribute__((address_space(3))) T*
+constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the 4-row blocks of a tile
+constexpr int F_TILE = psa_tiles::LT_TILE;  // bytes of one K or V tile (D = 128)
 
 
 #define TILE_SYNC()                         \
@@ -566,87 +564,20 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
   const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
 
-  // ---- lane-invariant addressing --------------------------------------------------------------------
-  // fetch: lane (q = lane/16, pos = lane%16) of block n of a 16-row group writes row q of that block at
-  // position pos, i.e. tile slot 4q + n, chunk pos ^ q
-  const int fq = lane >> 4;
-  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
-  // K operand of k-step kk: tile slot l32 (+32) = block 4*(l32>>4) + (l32&3), row (l32>>2)&3, chunk 2kk + hh
-  // -> k_off[kk & 1] + 64 * (kk >> 1)   (+ 8 blocks for the second 32 keys)
-  uint32_t k_off[2];
-  {
-    const int q = (l32 >> 2) & 3;
-    const int base = (4 * (l32 >> 4) + (l32 & 3)) * F_ISTR + q * 256;
-    k_off[0] = (uint32_t)(base + ((hh ^ q) * 16));
-    k_off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
-  }
-  // V operand (transposing read).  Inside a block of 16 lanes, lane i supplies the address of 4 channels
-  // (4*(i%4)..) of key i/4 and receives channel i of the block's 4 keys.  Lane block bl covers channels
-  // 32*db + 16*(bl&1).. and keys 16*cg + 8*s + 4*(bl>>1)..  (s = first / second half of the operand):
-  // tile slot 16*cg + 4*qq + n with qq = 2s + (bl>>1), n = i/4 -> block 4*cg + n, row qq
-  // -> v_off[s] + 64 * db + 4 * F_ISTR * cg
-  uint32_t v_off[2];
-  {
-    const int i16 = lane & 15, bl = lane >> 4;
-    const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int qq = 2 * s + (bl >> 1);
-      v_off[s] = (uint32_t)(n * F_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
-    }
-  }
+  // ---- lane-invariant addressing (tile layout: psa_tiles.h) -------------------------------------------
+  const uint32_t f_chunk = psa_tiles::lt_fetch_chunk(lane);
+  uint32_t k_off[2], v_off[2];
+  psa_tiles::lt_row_operand(l32, hh, k_off);  // K rows l32 (+32): k_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
+  psa_tiles::lt_tr_operand(lane, v_off);      // V^T: v_off[s] + 64 * db + 4 * F_ISTR * cg
 
-  // Where tile t comes from: base pointers and row strides (uniform), and for every 16-row group this
-  // wave fetches the first of the lane's 4 consecutive source rows.
-  struct TileSrc {
-    const char *kbase, *vbase;
-    uint32_t kstr, vstr;
-    int lim;          // last valid row when the tile may run past the sequence end, else INT_MAX
-    int src0[G16];
-  };
-  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) {
-    const u32x2 dd = tdesc[t];
-    const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd[0]);
-    const uint32_t d1 = __builtin_amdgcn_readfirstlane(dd[1]);
-    const int lv = d0 & 3, nvalid = (d0 >> 3) & 127, lt = d0 >> 10;
-    const int cnt = d1 >> 16;
-    const uint16_t* lids = ids + (d1 & 0xffff);
-    const int sbs_log2 = P_bn_log2 - lv;
-    const int lm1 = lv > 0 ? lv - 1 : 0;
-    const int64_t pool_off = (BHkv * (P_npad - (P_npad >> lm1)) + bhk * (P_npad >> lv)) * (D * 2);
-    a.kbase = lv == 0 ? kb0 : (const char*)P_kp + pool_off;
-    a.vbase = lv == 0 ? vb0 : (const char*)P_vp + pool_off;
-    a.kstr = lv == 0 ? P_k_strb : (uint32_t)(D * 2);
-    a.vstr = lv == 0 ? P_v_strb : (uint32_t)(D * 2);
-    const bool ragged = nvalid < TK;  // some slots are empty: clamp them onto real rows (their logits are masked)
-    a.lim = (ragged && lv == 0) ? P_L - 1 : 0x7fffffff;
-#pragma unroll
-    for (int gi = 0; gi < G16; ++gi) {
-      const int g = (lt << 6) + (wave * G16 + gi) * 16 + fq * 4;
-      int bi = g >> sbs_log2;
-      if (ragged) bi = bi < cnt - 1 ? bi : cnt - 1;
-      a.src0[gi] = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
-    }
-  };
-  // 4 rows per instruction go to block 4*g16 + n of the buffer at lds_byte
+  psa_tiles::KvSource kvs;
+  kvs.k0 = kb0; kvs.v0 = vb0; kvs.kp = (const char*)P_kp; kvs.vp = (const char*)P_vp;
+  kvs.k_strb = P_k_strb; kvs.v_strb = P_v_strb;
+  kvs.BHkv = BHkv; kvs.bhk = bhk; kvs.npad = P_npad; kvs.bn_log2 = P_bn_log2; kvs.L = P_L;
+  using TileSrc = psa_tiles::TileSrc<G16>;
+  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) { psa_tiles::lt_tile_src<G16>(kvs, tdesc, ids, t, wave, lane, a); };
   auto issue_rows = [&](const char* base, uint32_t str, int lim, const int (&src0)[G16], int lds_byte) __attribute__((always_inline)) {
-#pragma unroll
-    for (int gi = 0; gi < G16; ++gi) {
-      const int blk = (wave * G16 + gi) * 4;
-      if (lim == 0x7fffffff) {
-        // the usual case: the uniform base pointer steps from row to row, the lane offset stays
-        const uint32_t off = (uint32_t)src0[gi] * str + f_chunk;
-#pragma unroll
-        for (int n = 0; n < 4; ++n)
-          __builtin_amdgcn_global_load_lds(base + (uint64_t)(n * str) + off, (PSA_LDS(void))(smem + lds_byte + (blk + n) * F_ISTR), 16, 0, 0);
-      } else {
-#pragma unroll
-        for (int n = 0; n < 4; ++n) {
-          const int src = src0[gi] + n < lim ? src0[gi] + n : lim;
-          __builtin_amdgcn_global_load_lds(base + ((uint32_t)src * str + f_chunk), (PSA_LDS(void))(smem + lds_byte + (blk + n) * F_ISTR), 16, 0, 0);
-        }
-      }
-    }
+    psa_tiles::lt_issue_rows<G16>(smem + lds_byte, base, str, lim, src0, wave, f_chunk);
   };
 
   f32x16 acc[DB];

@@ -164,4 +164,116 @@ __device__ __forceinline__ int64_t pool_row_offset(int lv, int64_t BHkv, int64_t
   return BHkv * (npad - (npad >> lm1)) + bhk * (npad >> lv);
 }
 
+// ------------------------------------------------------------------------------------------------------
+// LDS tile layout of the head-dim-128 kernels (64 rows x 256 bytes, filled by global_load_lds_dwordx4).
+//   * a tile is 16 blocks of 4 rows, blocks LT_ISTR = 1024 + 64 bytes apart (one copy instruction per block:
+//     64 lanes x 16 bytes land at consecutive LDS addresses);
+//   * row q of a block stores its 16-byte chunks XOR-swizzled: chunk c sits at position c ^ q (applied on the
+//     global side: a lane fetches the chunk that belongs at its LDS position);
+//   * inside each group of 16 rows the rows are stored 4x4-transposed: block n, row q holds tile row 4q + n,
+//     so the 4 rows a lane fetches are 4 CONSECUTIVE tile rows.
+// Padding and swizzle make the 128-bit row reads and the transposing reads bank-conflict free, and both only
+// touch the low bits of the chunk index, so every operand address is lane base + immediate.
+// ------------------------------------------------------------------------------------------------------
+constexpr int LT_ISTR = 1024 + 64;
+constexpr int LT_TILE = 16 * LT_ISTR;
+
+#define PSA_LDS(T) __attribute__((address_space(3))) T*
+
+// copy side: byte offset of the chunk a lane fetches, and the first of its 4 tile rows inside a 16-row group
+__device__ __forceinline__ uint32_t lt_fetch_chunk(int lane) { return (uint32_t)(((lane & 15) ^ (lane >> 4)) * 16); }
+__device__ __forceinline__ int lt_fetch_row(int lane) { return (lane >> 4) * 4; }
+
+// MFMA row operand (A: 32 tile rows x 16 channels) of k-step kk for tile row `row`, hh = lane / 32:
+// off[kk & 1] + 64 * (kk >> 1)
+__device__ __forceinline__ void lt_row_operand(int row, int hh, uint32_t (&off)[2]) {
+  const int q = (row >> 2) & 3;
+  const int base = (4 * (row >> 4) + (row & 3)) * LT_ISTR + q * 256;
+  off[0] = (uint32_t)(base + ((hh ^ q) * 16));
+  off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
+}
+
+// MFMA transposed operand (A: 32 channels x 16 tile rows) through ds_read_b64_tr_b16.  Inside a block of 16
+// lanes, lane i supplies the address of 4 channels (4*(i%4)..) of row i/4 and receives channel i of the
+// block's 4 rows.  Lane block bl covers channels 32*db + 16*(bl&1).. and rows 16*grp + 8*s + 4*(bl>>1)..
+// (s = first / second half of the operand): off[s] + 64 * db + 4 * LT_ISTR * grp.  The row order inside the
+// operand equals the order in which the 32x32 MFMA accumulator layout hands 8 consecutive registers to a lane.
+__device__ __forceinline__ void lt_tr_operand(int lane, uint32_t (&off)[2]) {
+  const int i16 = lane & 15, bl = lane >> 4;
+  const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int qq = 2 * s + (bl >> 1);
+    off[s] = (uint32_t)(n * LT_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
+  }
+}
+
+// Where the K / V rows of a tile come from (uniform per workgroup).
+struct KvSource {
+  const char *k0, *v0;      // level 0: this (batch, kv head) slice of K and V
+  const char *kp, *vp;      // pooled buffers (all batches, heads and levels)
+  uint32_t k_strb, v_strb;  // level-0 row strides in bytes
+  int64_t BHkv, bhk, npad;
+  int bn_log2, L;
+};
+
+// Source of tile t for the wave that copies the 16-row groups wave*G16 .. wave*G16 + G16 - 1
+template <int G16>
+struct TileSrc {
+  const char *kbase, *vbase;
+  uint32_t kstr, vstr;
+  int lim;        // last valid row when the tile may run past the sequence end, else INT_MAX
+  int src0[G16];  // first of the lane's 4 consecutive source rows, per group
+};
+
+template <int G16>
+__device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tdesc, const uint16_t* ids, int t, int wave, int lane,
+                                            TileSrc<G16>& a) {
+  const u32x2 dd = tdesc[t];
+  const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd[0]);
+  const uint32_t d1 = __builtin_amdgcn_readfirstlane(dd[1]);
+  const int lv = d0 & 3, nvalid = (d0 >> 3) & 127, lt = d0 >> 10;
+  const int cnt = d1 >> 16;
+  const uint16_t* lids = ids + (d1 & 0xffff);
+  const int sbs_log2 = kv.bn_log2 - lv;
+  const int lm1 = lv > 0 ? lv - 1 : 0;
+  const int64_t pool_off = (kv.BHkv * (kv.npad - (kv.npad >> lm1)) + kv.bhk * (kv.npad >> lv)) * 256;
+  a.kbase = lv == 0 ? kv.k0 : kv.kp + pool_off;
+  a.vbase = lv == 0 ? kv.v0 : kv.vp + pool_off;
+  a.kstr = lv == 0 ? kv.k_strb : 256u;
+  a.vstr = lv == 0 ? kv.v_strb : 256u;
+  const bool ragged = nvalid < TK;  // some slots are empty: clamp them onto real rows (their logits are masked)
+  a.lim = (ragged && lv == 0) ? kv.L - 1 : 0x7fffffff;
+#pragma unroll
+  for (int gi = 0; gi < G16; ++gi) {
+    const int g = (lt << 6) + (wave * G16 + gi) * 16 + lt_fetch_row(lane);
+    int bi = g >> sbs_log2;
+    if (ragged) bi = bi < cnt - 1 ? bi : cnt - 1;
+    a.src0[gi] = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
+  }
+}
+
+// Copies this wave's groups of one tile: 4 rows per instruction go to block 4*g16 + n of the tile at `dst`.
+template <int G16>
+__device__ __forceinline__ void lt_issue_rows(unsigned char* dst, const char* base, uint32_t str, int lim, const int (&src0)[G16],
+                                              int wave, uint32_t f_chunk) {
+#pragma unroll
+  for (int gi = 0; gi < G16; ++gi) {
+    const int blk = (wave * G16 + gi) * 4;
+    if (lim == 0x7fffffff) {
+      // the usual case: the uniform base pointer steps from row to row, the lane offset stays
+      const uint32_t off = (uint32_t)src0[gi] * str + f_chunk;
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+        __builtin_amdgcn_global_load_lds(base + (uint64_t)(n * str) + off, (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        const int src = src0[gi] + n < lim ? src0[gi] + n : lim;
+        __builtin_amdgcn_global_load_lds(base + ((uint32_t)src * str + f_chunk), (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
+      }
+    }
+  }
+}
+
 }  // namespace psa_tiles
