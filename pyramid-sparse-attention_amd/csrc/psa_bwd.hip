@@ -761,6 +761,78 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int s
 }
 
 // ------------------------------------------------------------------------------------------------------
+// Longest-columns-first order for the dK/dV walk.  A workgroup's work is the number of q-blocks that retain its
+// kv-block at its level, which varies a lot (a few key blocks are kept by every query block); issuing the
+// workgroups by decreasing work removes the tail of the launch.  Results do not depend on the order.
+// ------------------------------------------------------------------------------------------------------
+constexpr int COL_BINS = 2048;
+
+// one workgroup per (kv head, kv-block): per-level counts over the column -> cost of each of its slots
+__global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int slots_per_block, int32_t* cost) {
+  __shared__ int s_n[4];
+  const int J = blockIdx.x, bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  const int n_rep = p.Hq / p.Hkv, Mq = p.Mq, bn_log2 = p.bn_log2;
+  if (threadIdx.x < 4) s_n[threadIdx.x] = 0;
+  __syncthreads();
+  int n[4] = {0, 0, 0, 0};
+  for (int e = threadIdx.x; e < n_rep * Mq; e += 256) {
+    const int hl = e / Mq, I = e % Mq;
+    const int h = hk * n_rep + hl;
+    int level = load_map(p.map, (((int64_t)b * p.Hq + h) * Mq + I) * p.Nk + J, p.map_elem);
+    if (p.causal) {
+      const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << bn_log2) - 1) >> bn_log2);
+      if (J >= ce) level = 0;
+    }
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) n[lv] += level == (1 << lv);
+  }
+#pragma unroll
+  for (int lv = 0; lv < 4; ++lv)
+    if (n[lv]) atomicAdd(&s_n[lv], n[lv]);
+  __syncthreads();
+  if ((int)threadIdx.x < slots_per_block) {
+    int lv, part;
+    decode_slot((int)threadIdx.x, bn_log2, lv, part);
+    const int c = s_n[lv];
+    cost[((int64_t)bhk * p.Nk + J) * slots_per_block + threadIdx.x] = c < COL_BINS - 1 ? c : COL_BINS - 1;
+  }
+}
+
+// one workgroup: counting sort of all workgroup ids by decreasing cost
+__global__ __launch_bounds__(256) void psa_bwd_colsort_kernel(const int32_t* cost, int total, int32_t* order) {
+  __shared__ int hist[COL_BINS];
+  __shared__ int part[256];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < COL_BINS; i += 256) hist[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < total; i += 256) atomicAdd(&hist[cost[i]], 1);
+  __syncthreads();
+  constexpr int PER = COL_BINS / 256;  // thread i owns the bins COL_BINS-1-PER*i .. COL_BINS-PER-PER*i
+  int c[PER], sum = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    c[j] = hist[COL_BINS - 1 - (tid * PER + j)];
+    sum += c[j];
+  }
+  part[tid] = sum;
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
+    const int add = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += add;
+    __syncthreads();
+  }
+  int run = part[tid] - sum;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    hist[COL_BINS - 1 - (tid * PER + j)] = run;
+    run += c[j];
+  }
+  __syncthreads();
+  for (int i = tid; i < total; i += 256) order[atomicAdd(&hist[cost[i]], 1)] = i;
+}
+
+// ------------------------------------------------------------------------------------------------------
 // dK/dV column walk, head dim 128: Q and dO rows are copied from global memory straight into LDS (double
 // buffered, one barrier per step of 64 query rows) in the padded + swizzled row-major tile layout of the forward
 // kernel; the row operands (S = Q K^T, dP = dO V^T) are 128-bit LDS reads and the transposed operands
@@ -769,7 +841,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int s
 constexpr int B_ISTR = LT_ISTR;  // bytes between the 4-row blocks of a tile
 constexpr int B_TILE = LT_TILE;  // 64 rows x 256 bytes, padded
 
-__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, int slots_per_block) {
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, int slots_per_block, const int32_t* order) {
   constexpr int D = 128, KK = D / 16, DB = D / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   // stage s: Q tile at 2*s*B_TILE, dO tile at (2*s + 1)*B_TILE
@@ -778,9 +850,11 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
   uint32_t* qlist = (uint32_t*)(s_del + 128);  // [n_rep * Mq]  (head in group << 16 | q-block)
   __shared__ int s_nq;
 
-  const int slot = blockIdx.x % slots_per_block;
-  const int J = blockIdx.x / slots_per_block;
-  const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  // flat workgroup id = ((b * Hkv + kv head) * Nk + kv-block) * slots_per_block + slot, optionally re-ordered
+  const int wg = order != nullptr ? order[blockIdx.x] : (int)blockIdx.x;
+  const int slot = wg % slots_per_block;
+  const int J = (wg / slots_per_block) % p.Nk;
+  const int bhk = wg / (slots_per_block * p.Nk), b = bhk / p.Hkv, hk = bhk % p.Hkv;
   const int n_rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hh = lane >> 5;
@@ -798,7 +872,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
   }
   // waves = 2 key halves x 2 query halves.  With at most 32 keys only one key half works: alternate which
   // pair of waves that is from workgroup to workgroup, so that all four SIMDs of a CU get work.
-  const int flip = nkeys <= 32 ? (int)((blockIdx.x + blockIdx.y) & 1) : 0;
+  const int flip = nkeys <= 32 ? (int)(blockIdx.x & 1) : 0;
   const int kh = (wave & 1) ^ flip, qh = wave >> 1;
   const bool wave_active = key_valid > kh * 32;
 
@@ -1118,7 +1192,9 @@ extern "C" int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D,
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || L <= 0 || D <= 0 || block_n <= 0) return 0;
   const int64_t npad = (int64_t)((L + block_n - 1) / block_n) * block_n;
   const int64_t levels = (int64_t)B * Hkv * D * (npad + npad / 2 + npad / 4 + npad / 8);
-  return (2 * levels + 2 * (int64_t)B * Hq * L) * (int64_t)sizeof(float);
+  // + cost and order of the dK/dV workgroups (at most 8 slots per kv-block)
+  const int64_t n_wg = (int64_t)B * Hkv * ((L + block_n - 1) / block_n) * 8;
+  return (2 * levels + 2 * (int64_t)B * Hq * L + 2 * n_wg) * (int64_t)sizeof(float);
 }
 
 extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool, const void* map,
@@ -1206,21 +1282,34 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   {
     const int spb = slots_of(block_n);
     const int n_rep = Hq / Hkv;
-    dim3 grid((unsigned)(Nk * spb), (unsigned)(B * Hkv));
-    auto launch = [&](auto kern, size_t stage_bytes) -> int {
-      size_t shmem = stage_bytes + 128 * sizeof(float) + (size_t)n_rep * Mq * 4;
-      const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
-      if (shmem < red) shmem = red;
-      if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-      if (shmem > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-        return PSA_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, grid, dim3(256), shmem, st, p, spb);
-      return PSA_OK;
-    };
-    int rc = D == 128 ? launch(psa_bwd_dkdv128_kernel, (size_t)4 * B_TILE + 128 * sizeof(float))
-                      : launch(psa_bwd_dkdv_kernel<64>, KvSmem<64>::STAGE_BYTES);
-    PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
-    rc = psa_check_launch("psa_bwd (dK/dV)");
+    const int64_t n_wg = (int64_t)B * Hkv * Nk * spb;
+    PSA_REQUIRE(n_wg < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    size_t shmem = (D == 128 ? (size_t)4 * LT_TILE + 256 * sizeof(float) : KvSmem<64>::STAGE_BYTES + 128 * sizeof(float)) +
+                   (size_t)n_rep * Mq * 4;
+    const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
+    if (shmem < red) shmem = red;
+    PSA_REQUIRE(shmem <= 160 * 1024, PSA_ERR_UNSUPPORTED, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
+    if (D == 128) {
+      // longest columns first (needs a level map; the order lives behind lse2 in the workspace)
+      int32_t* order = nullptr;
+      if (map != nullptr && n_wg > 32) {
+        int32_t* cost = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
+        order = cost + n_wg;
+        hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, spb, cost);
+        if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
+        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(256), 0, st, cost, (int)n_wg, order);
+        if (int e = psa_check_launch("psa_bwd (column order)")) return e;
+      }
+      PSA_REQUIRE(hipFuncSetAttribute((const void*)psa_bwd_dkdv128_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) == hipSuccess,
+                  PSA_ERR_LAUNCH, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
+      hipLaunchKernelGGL(psa_bwd_dkdv128_kernel, dim3((unsigned)n_wg), dim3(256), shmem, st, p, spb, order);
+    } else {
+      PSA_REQUIRE(shmem <= 48 * 1024 || hipFuncSetAttribute((const void*)psa_bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                            (int)shmem) == hipSuccess,
+                  PSA_ERR_LAUNCH, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
+      hipLaunchKernelGGL(psa_bwd_dkdv_kernel<64>, dim3((unsigned)(Nk * spb), (unsigned)(B * Hkv)), dim3(256), shmem, st, p, spb);
+    }
+    const int rc = psa_check_launch("psa_bwd (dK/dV)");
     if (rc != PSA_OK) return rc;
   }
   // 4. un-pool
