@@ -31,6 +31,18 @@ WORKLOADS = {
     "c1": dict(name="small B1 H2 N4096 D64 blk64 thresholdbound ~80% sparsity",
                B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80),
 }
+WORKLOADS.update({
+    # BASELINE.json configs[2]: CogVideoX-5B joint text + video attention (text blocks last, always level 1)
+    "c3": dict(name="cogvideox-5b B2 H48 N17776 (17550 video + 226 text) D64 bf16 blk128 thresholdbound ~85% sparsity",
+               B=2, H=48, grid=(13, 30, 45), D=64, bm=128, bn=128, tn=32, sparsity=0.85, text=226),
+    # BASELINE.json configs[3]: training step = forward with lse + backward (dQ, dK, dV)
+    "c4": dict(name="training step B1 H12 N32760 D128 bf16 blk128 thresholdbound ~85% sparsity, dO ~ N(0, 0.02)",
+               B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.85, kind="train"),
+    # BASELINE.json configs[4]: causal GQA prefill at the Qwen2.5-VL-7B decoder shape
+    "c5": dict(name="qwen2.5-vl-7b causal prefill B1 Hq28 Hkv4 N32768 (1024 text + 16x44x44 vision) D128 bf16 blk128 "
+                    "energybound ~80% sparsity over the lower triangle",
+               B=1, H=28, Hkv=4, grid=(16, 44, 44), D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal"),
+})
 WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
 
 
@@ -56,6 +68,95 @@ def time_gpu(fn, iters, warm=3):
     torch.cuda.synchronize()
     ts = sorted(a.elapsed_time(b) for a, b in evs)
     return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
+    """The training-step and causal-prefill configurations: same JSON layout, their own stages."""
+    B, H, D, bm, bn = w["B"], w["H"], w["D"], w["bm"], w["bn"]
+    Hkv = w.get("Hkv", H)
+    text = w.get("text", 0)
+    causal = w["kind"] == "causal"
+    q, k, v = make_qkv(B, H, Hkv, w["grid"], D, seed=args.seed, device=dev, text_tokens=text, text_first=causal)
+    L = q.shape[2]
+    it = max(5, min(args.steps, 30))
+    stages = {}
+    if causal:
+        # antidiagonal estimate -> causal level map (energy bound scaled to the sparsity target) -> causal GQA forward
+        base = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
+        est = ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True)
+        lo, hi = 0.05, 1.25
+        for _ in range(16):
+            tau = 0.5 * (lo + hi)
+            ratios = {lv: ((a * tau, b * tau) if lv else (0.8 * tau, 1.0)) for lv, (a, b) in base.items()}
+            mp = ops.level_map_qwen(est, ratios, text, "energybound", block_size=bm, causal=True, map_dtype=torch.int8)
+            dens = float(ops.density(mp, causal=True)[-1])
+            lo, hi = (tau, hi) if 1 - dens > w["sparsity"] else (lo, tau)
+
+        def step():
+            e = ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True)
+            m = ops.level_map_qwen(e, ratios, text, "energybound", block_size=bm, causal=True, map_dtype=torch.int8)
+            return ops.sparse_attention_fwd(q, k, v, m, bm, bn, causal=True)
+
+        stages["estimate_xattn"], _ = time_gpu(lambda: ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True), it)
+        stages["level_map"], _ = time_gpu(lambda: ops.level_map_qwen(est, ratios, text, "energybound", block_size=bm, causal=True,
+                                                                    map_dtype=torch.int8), it)
+        kp, vp = ops.pool_kv(k, v, bn)
+        stages["pool"], _ = time_gpu(lambda: ops.pool_kv(k, v, bn), it)
+        t_fwd, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, causal=True, pools=(kp, vp)), it)
+        stages["sparse_fwd"] = t_fwd
+        dense_flops = 4.0 * L * L * D * H * B / 2  # lower triangle
+    else:
+        km, kn = bm // 4, bn // 4
+        off_q = sample_offsets(B, H, bm, km, args.seed + 10, device=dev)
+        off_k = sample_offsets(B, Hkv, bn, kn, args.seed + 11, device=dev)
+        scores = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
+        lo, hi = 0.05, 1.25
+        for _ in range(16):
+            tau = 0.5 * (lo + hi)
+            mp = ops.level_map(scores, scaled_ratios(tau), text, "thresholdbound", blocksize=bn, compute_tile=w["tn"], map_dtype=torch.int8)
+            dens = float(ops.density(mp)[-1])
+            lo, hi = (tau, hi) if 1 - dens > w["sparsity"] else (lo, tau)
+        g = torch.Generator(device="cpu").manual_seed(args.seed + 5)
+        dout = (torch.randn(q.shape, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        out, lse, pools = ops.sparse_attention_fwd(q, k, v, mp, bm, bn, return_lse=True)
+
+        def step():
+            o, l, pl = ops.sparse_attention_fwd(q, k, v, mp, bm, bn, return_lse=True)
+            return ops.sparse_attention_bwd(q, k, v, mp, o, dout, l, bm, bn, pools=pl)
+
+        t_fwd, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, return_lse=True), it)
+        stages["sparse_fwd_with_pooling"] = t_fwd
+        stages["backward"], _ = time_gpu(lambda: ops.sparse_attention_bwd(q, k, v, mp, out, dout, lse, bm, bn, pools=pools), it)
+        dense_flops = 4.0 * L * L * D * H * B * 3.5  # forward + backward of dense attention
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_step = e0.elapsed_time(e1) / args.steps
+    density = float(ops.density(mp, causal=causal)[-1])
+    fwd_flops = 4.0 * L * L * D * H * B * density * (0.5 if causal else 1.0)
+    stages = {kk: round(vv, 4) for kk, vv in stages.items()}
+    stages["step"] = round(ms_step, 4)
+    return {
+        "metric": METRIC, "value": round(dense_flops / (ms_step * 1e-3) / 1e12, 2),
+        "unit": "effective TFLOP/s (dense-equivalent flops of the step / step time)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seeded smooth 3-D field + noise, logit std ~3; text tokens i.i.d. N(0,1))",
+        "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
+                   "sparsity": round(1 - density, 4)},
+        "stages_ms": stages,
+        "roofline": {"kernel": "psa_fwd_d128_kernel", "bound": "mfma",
+                     "achieved": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": fwd_flops, "avg_launch_ms": round(t_fwd_avg, 4)},
+        "cpu_baseline": None,
+    }
 
 
 def main():
@@ -88,8 +189,12 @@ def main():
     w = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if w.get("kind") in ("train", "causal"):
+        print(json.dumps(run_other(args, w, torch, ops, make_qkv, sample_offsets, dev)))
+        return
     B, H, D, bm, bn, tn = w["B"], w["H"], w["D"], w["bm"], w["bn"], w["tn"]
-    q, k, v = make_qkv(B, H, H, w["grid"], D, seed=args.seed, device=dev)
+    text = w.get("text", 0)
+    q, k, v = make_qkv(B, H, H, w["grid"], D, seed=args.seed, device=dev, text_tokens=text)
     L = q.shape[2]
     Mq, Nk = -(-L // bm), -(-L // bn)
     km, kn = bm // 4, bn // 4
@@ -101,7 +206,7 @@ def main():
     lo, hi = 0.05, 1.25
     for _ in range(18):
         tau = 0.5 * (lo + hi)
-        m = ops.level_map(scores, scaled_ratios(tau), 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
+        m = ops.level_map(scores, scaled_ratios(tau), text, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
         dens = float(ops.density(m)[-1])
         if 1 - dens > w["sparsity"]:
             lo = tau
@@ -113,7 +218,7 @@ def main():
 
     def layer():
         # estimate -> level map -> pooling -> forward
-        o, mp = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+        o, mp = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, "thresholdbound", bm, bn, tn, return_map=True, text_length=text)
         state.update(mp=mp, o=o)
         return o
 
@@ -142,7 +247,7 @@ def main():
     it = max(10, min(args.steps, 100))
     t_pool, _ = time_gpu(lambda: ops.pool_kv(k, v, bn), it)
     t_est, _ = time_gpu(lambda: ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn), it)
-    t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
+    t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
     out_buf = torch.empty_like(q)
     t_fwd_med, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf), it)
     t_dense = t_sdpa = None
@@ -183,7 +288,7 @@ def main():
         oqc, okc = off_q[:, heads].cpu(), off_k[:, heads].cpu()
         t0c = time.perf_counter()
         s_c = O.estimate_sampled(qc, kc, bm, bn, oqc, okc)
-        O.level_map(s_c.numpy(), ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn)
+        O.level_map(s_c.numpy(), ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn)
         t_front = time.perf_counter() - t0c  # pooling is inside blockwalk
         t1c = time.perf_counter()
         O.psa_attention_blockwalk(qc, kc, vc, mc, bm, bn, qblocks=qblocks)

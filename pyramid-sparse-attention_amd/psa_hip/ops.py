@@ -327,6 +327,7 @@ def psa_layer_fwd(
     sm_scale: Optional[float] = None,
     level_cap: Optional[torch.Tensor] = None,
     return_map: bool = False,
+    text_length: int = 0,
 ):
     """estimate -> level map -> pooled K/V -> sparse attention, non-causal, no gradient: the four stages
     on the current stream with a dense int8 level map in between (no index-list round trip).  Running the
@@ -337,7 +338,7 @@ def psa_layer_fwd(
     keep_m, keep_n = block_m // 4, block_n // 4
     sm_scale = qb.shape[-1] ** -0.5 if sm_scale is None else float(sm_scale)
     scores = estimate_sampled(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, sm_scale)
-    mp = level_map(scores, mask_ratios, 0, mode, blocksize=block_n, compute_tile=tile_n, map_dtype=torch.int8)
+    mp = level_map(scores, mask_ratios, text_length, mode, blocksize=block_n, compute_tile=tile_n, map_dtype=torch.int8)
     if level_cap is not None:
         mp = map_min_cap(mp, level_cap)
     kp, vp = pool_kv(kb, vb, block_n)
