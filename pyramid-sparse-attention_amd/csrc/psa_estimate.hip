@@ -376,26 +376,34 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
 }
 
 // one workgroup per (b, h, query group): Po[i, :] from R^T and m.
-// A wave reads 64/keep_m key groups at a time: lane l holds row l % keep_m of key group j0 + l / keep_m,
-// i.e. every keep_m-lane segment reads one contiguous run of the workspace; the maximum over the
-// group's rows is a butterfly inside the segment.
+// A lane reads 4 consecutive rows (16 bytes) of one key group, keep_m/4 neighbouring lanes cover the group's
+// rows (one contiguous run of the workspace), a wave 256/keep_m key groups per load; the maximum over the
+// group's rows is an in-lane maximum plus a butterfly over those lanes.
 __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
   extern __shared__ float s_e[];  // [n_d] un-normalised Po row
   __shared__ float s_part[4];
   const int i = blockIdx.x, bh = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int keep_m = 1 << p.keep_m_log2;
-  const int row = lane & (keep_m - 1), sub = lane >> p.keep_m_log2;
-  const int per_iter = 64 >> p.keep_m_log2;  // key groups per wave iteration
-  const int r0 = i * keep_m;
-  float m = -INFINITY;
-  for (int ks = 0; ks < p.ksplit; ++ks) m = fmaxf(m, p.mrow[((int64_t)bh * p.ksplit + ks) * p.Ms_pad + r0 + row]);
-  const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0 + row;
+  const int lpg_log2 = p.keep_m_log2 - 2;            // lanes per key group
+  const int quad = lane & ((1 << lpg_log2) - 1), sub = lane >> lpg_log2;
+  const int per_iter = 64 >> lpg_log2;               // key groups per wave iteration
+  const int r0 = (i << p.keep_m_log2) + quad * 4;
+  f32x4 m = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+  for (int ks = 0; ks < p.ksplit; ++ks) {
+    const f32x4 x = *(const f32x4*)(p.mrow + ((int64_t)bh * p.ksplit + ks) * p.Ms_pad + r0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m[e] = fmaxf(m[e], x[e]);
+  }
+  const float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + r0;
   for (int j0 = wave * per_iter; j0 < p.n_d; j0 += 4 * per_iter) {
     const int j = j0 + sub;
-    float v = j < p.n_d ? rt[(int64_t)j * p.Ms_pad] - m : -INFINITY;
-    for (int o = keep_m >> 1; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    if (row == 0 && j < p.n_d) s_e[j] = fast_exp2(v);
+    float v = -INFINITY;
+    if (j < p.n_d) {
+      const f32x4 x = *(const f32x4*)(rt + (int64_t)j * p.Ms_pad);
+      v = fmaxf(fmaxf(x[0] - m[0], x[1] - m[1]), fmaxf(x[2] - m[2], x[3] - m[3]));
+    }
+    for (int o = (1 << lpg_log2) >> 1; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    if (quad == 0 && j < p.n_d) s_e[j] = fast_exp2(v);
   }
   __syncthreads();
   // row sum in a fixed order: per-thread strided partials, wave butterfly, four wave partials
