@@ -49,6 +49,9 @@ def run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed, lmap=None):
         (1, 2, 2, 320, 64, 64, 64),
         (1, 1, 1, 400, 128, 128, 32),
         (1, 1, 1, 300, 64, 128, 64),
+        (1, 2, 2, 330, 128, 64, 64),      # head dim 128 with 64-row q-blocks
+        (1, 1, 1, 67, 128, 128, 128),     # a single, partly filled block
+        (1, 3, 1, 200, 128, 128, 64),     # GQA with three query heads per kv head
     ],
 )
 @pytest.mark.parametrize("causal", [False, True])
@@ -81,6 +84,21 @@ def test_bwd_all_ones_matches_sdpa_autograd():
     out, lse, _ = ops.sparse_attention_fwd(qd, kd, vd, None, 128, 128, return_lse=True)
     dq, dk, dv = ops.sparse_attention_bwd(qd, kd, vd, None, out, dod, lse, 128, 128)
     assert max(rel_l2(dq, qq.grad), rel_l2(dk, kk.grad), rel_l2(dv, vv.grad)) <= REL_L2
+
+
+def test_bwd_strided_bf16_head_dim_128():
+    """q, k, v, dO in [B,L,H,D] memory layout (views), gradients returned densely."""
+    from psa_hip import ops
+
+    B, H, L, D = 1, 2, 390, 128
+    q, k, v, do = (rnd(B, L, H, D, seed=s) for s in (21, 22, 23, 24))
+    lmap = random_map(B, H, 4, 4, 5)
+    qd, kd, vd, dod = (t.to(dev()).transpose(1, 2) for t in (q, k, v, do))
+    md = torch.from_numpy(lmap).to(dev())
+    out, lse, pools = ops.sparse_attention_fwd(qd, kd, vd, md, 128, 128, return_lse=True)
+    dq, dk, dv = ops.sparse_attention_bwd(qd, kd, vd, md, out, dod, lse, 128, 128, pools=pools)
+    rq, rk, rv = O.psa_backward_dense(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), lmap, do.transpose(1, 2), 128, 128)
+    assert max(rel_l2(dq, rq), rel_l2(dk, rk), rel_l2(dv, rv)) <= REL_L2
 
 
 def test_legacy_factory_autograd():

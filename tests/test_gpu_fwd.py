@@ -42,6 +42,11 @@ def run_case(B, Hq, Hkv, L, D, bm, bn, causal, seed, lmap=None, p=(0.35, 0.2, 0.
         (1, 2, 2, 600, 128, 128, 64),
         (1, 4, 2, 512, 128, 128, 128),    # GQA
         (1, 1, 1, 100, 64, 64, 32),
+        (1, 2, 2, 700, 128, 64, 64),      # head dim 128 with 64-row q-blocks (2 waves per workgroup)
+        (1, 2, 1, 333, 128, 64, 32),
+        (1, 2, 2, 130, 128, 64, 128),
+        (1, 1, 1, 3, 128, 128, 128),      # shorter than one run of 4 tile rows
+        (1, 1, 1, 65, 128, 128, 128),
     ],
 )
 @pytest.mark.parametrize("causal", [False, True])
@@ -121,6 +126,22 @@ def test_fwd_strided_and_fp32_inputs():
     ref, _ = O.psa_attention_dense(qt.bfloat16(), kt.bfloat16(), vt.bfloat16(), lm, 128, 128)
     mx, mean = attn_errors(out, ref)
     assert mx <= MAX_ABS and mean <= MEAN_ABS
+
+
+def test_fwd_strided_bf16_head_dim_128():
+    """[B,L,H,D] memory layout passed as a [B,H,L,D] view: rows of a head are H*D elements apart."""
+    from psa_hip import ops
+
+    B, H, L, D = 1, 3, 700, 128
+    q, k, v = rnd(B, L, H, D, seed=14), rnd(B, L, H, D, seed=15), rnd(B, L, H, D, seed=16)
+    lm = random_map(B, H, 6, 6, 2)
+    qt, kt, vt = (t.to(dev()).transpose(1, 2) for t in (q, k, v))
+    assert not kt.is_contiguous()
+    for causal in (False, True):
+        out = ops.sparse_attention_fwd(qt, kt, vt, torch.from_numpy(lm).to(dev()), 128, 128, causal=causal)
+        ref, _ = O.psa_attention_dense(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), lm, 128, 128, causal=causal)
+        mx, mean = attn_errors(out, ref)
+        assert mx <= MAX_ABS and mean <= MEAN_ABS
 
 
 def test_fwd_errors():
