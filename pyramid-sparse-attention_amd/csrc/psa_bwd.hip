@@ -347,16 +347,16 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) 
   kvs.k_strb = (uint32_t)p.k_sl * 2u; kvs.v_strb = (uint32_t)p.v_sl * 2u;
   kvs.BHkv = (int64_t)p.B * p.Hkv; kvs.bhk = (int64_t)b * p.Hkv + hk; kvs.npad = p.npad;
   kvs.bn_log2 = bn_log2; kvs.L = L;
-  const uint32_t f_chunk = lt_fetch_chunk(lane);
+  const uint32_t f_chunk = lt_fetch_chunk<128>(lane);
   uint32_t r_off[2], t_off[2];
-  lt_row_operand(l32, hh, r_off);  // tile rows l32 (+32): r_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
-  lt_tr_operand(lane, t_off);      // K^T: t_off[s] + 64 * db + 4 * LT_ISTR * (16-key group)
+  lt_row_operand<128>(l32, hh, r_off);  // tile rows l32 (+32): r_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
+  lt_tr_operand<128>(lane, t_off);      // K^T: t_off[s] + 64 * db + 4 * LT_ISTR * (16-key group)
 
   auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
     TileSrc<G16> ts;
-    lt_tile_src<G16>(kvs, tdesc, ids, t, wave, lane, ts);
-    lt_issue_rows<G16>(smem + stage * LT_TILE, ts.kbase, ts.kstr, ts.lim, ts.src0, wave, f_chunk);
-    lt_issue_rows<G16>(smem + (2 + stage) * LT_TILE, ts.vbase, ts.vstr, ts.lim, ts.src0, wave, f_chunk);
+    lt_tile_src<128, G16>(kvs, tdesc, ids, t, wave, lane, ts);
+    lt_issue_rows<128, G16>(smem + stage * LT_TILE, ts.kbase, ts.kstr, ts.lim, ts.src0, wave, f_chunk);
+    lt_issue_rows<128, G16>(smem + (2 + stage) * LT_TILE, ts.vbase, ts.vstr, ts.lim, ts.src0, wave, f_chunk);
   };
 
   f32x16 acc[DB];
@@ -931,11 +931,11 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
   // ---- lane-invariant LDS addressing (tile layout: see the forward kernel) ---------------------------
   // copy: wave w fills the 16-row group w of both tiles; lane (fq = lane/16, pos = lane%16) of block n writes
   // row fq of that block, i.e. tile row 16w + 4fq + n, chunk pos ^ fq
-  const uint32_t f_chunk = lt_fetch_chunk(lane);
-  const int f_row = wave * 16 + lt_fetch_row(lane);
+  const uint32_t f_chunk = lt_fetch_chunk<128>(lane);
+  const int f_row = wave * 16 + lt_fetch_row<128>(lane);
   uint32_t r_off[2], t_off[2];
-  lt_row_operand(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
-  lt_tr_operand(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
+  lt_row_operand<128>(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
+  lt_tr_operand<128>(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll

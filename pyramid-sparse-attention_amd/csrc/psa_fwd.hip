@@ -1,28 +1,29 @@
 // Pyramid sparse attention forward (non-causal and causal) on bf16 MFMA.
 //
-// One workgroup per (batch, head, q-block of BM = 32*NW rows); every wave owns 32 query rows.
+// One workgroup per (batch, head, q-block of BM = 32*NW rows); every wave owns 32 query rows; two workgroups
+// per CU.
 //
-//  * The workgroup first compacts its row of the level map into four per-level lists of kv-block
-//    ids in LDS (ballot + popcount, ascending block order - deterministic) and a list of tile
-//    descriptors.
-//  * Work is a sequence of TILES of 64 pooled keys of one level: a level-l kv-block holds
-//    block_n/l pooled keys, so one tile is half a 128-key block, one 64-key block, or 64/(block_n/l)
-//    small blocks of the same level packed side by side.  All tiles therefore cost the same MFMA
-//    work whatever their level; only the last tile of a level can be partly empty.
-//  * K tile -> LDS as [key][d] (row pad 16 B), V tile -> LDS TRANSPOSED as [d][key] (row pad 8 B):
-//    the 4x8 register transpose is done with v_perm while staging, so that both MFMA operands are
-//    read from LDS with the contraction index contiguous.
+//  * The workgroup first compacts its row of the level map into four per-level lists of kv-block ids in LDS
+//    (ballot + popcount, ascending block order - deterministic) and a list of tile descriptors.
+//  * Work is a sequence of TILES of 64 pooled keys of one level: a level-l kv-block holds block_n/l pooled
+//    keys, so one tile is half a 128-key block, one 64-key block, or 64/(block_n/l) small blocks of the same
+//    level packed side by side.  All tiles therefore cost the same MFMA work whatever their level; only the
+//    last tile of a level can be partly empty.
+//  * K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4: no staging registers, no
+//    VALU work), both row-major, double buffered, in the padded + swizzled layout of psa_tiles.h.  K operands
+//    are 128-bit LDS reads; V operands come through ds_read_b64_tr_b16, which hands every lane 4 keys of one
+//    channel: exactly the A operand of O^T += V^T P^T, in the key order that the S^T accumulator layout gives
+//    P^T.  All operand addresses are lane base + immediate (the tile loop is unrolled by two for that).
 //  * The kernel computes the transposed problem  S^T = K Q^T  (32 keys x 32 queries per MFMA,
-//    v_mfma_f32_32x32x16_bf16) and  O^T += V^T P^T.  In the MFMA accumulator layout a lane then
-//    holds 16 keys of ONE query column: the softmax row max / row sum are in-lane reductions plus a
-//    single exchange between the two half-waves, and P^T is already in B-operand layout (the
-//    key<->slot permutation it implies is applied to the V^T reads, which is free).
-//  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m); the running maximum is
-//    only raised when it grows by more than 2^8 would overflow nothing (lazy rescaling), so most
-//    tiles skip the accumulator rescale.
-//  * One barrier per tile: while tile t is computed from one pair of LDS buffers, tile t+1 is written
-//    to the other pair and the global loads of tile t+2 are in flight; inside a tile the LDS operand
-//    reads run one MFMA step ahead.  Two workgroups per CU overlap one's softmax with the other's MFMAs.
+//    v_mfma_f32_32x32x16_bf16) and  O^T += V^T P^T.  In the MFMA accumulator layout a lane then holds 16 keys of
+//    ONE query column: the softmax row max / row sum are in-lane reductions plus a single exchange between the
+//    two half-waves (v_permlane32_swap), and P^T is already in B-operand layout.
+//  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m); the reference maximum is only raised
+//    when it lags by more than 2^8 (lazy rescaling), so most tiles skip the accumulator rescale.  Row sums add
+//    the bf16-ROUNDED probabilities (v_dot2_f32_bf16): numerator and denominator use the same values.
+//  * One barrier per tile: copy of tile t+1 in flight | QK(t) | softmax(t) | PV(t) | barrier.
+//  * Rows are issued in groups (group g on XCD g mod 8, a few heads per phase of 8 groups) and, with the
+//    optional workspace, longest first inside a group.
 //
 // Roofline: MFMA-bound; 4*BM*64*D flops per tile.
 #include <type_traits>
@@ -52,454 +53,7 @@ struct FwdParams {
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
 };
 
-template <int D>
-struct Smem {
-  static constexpr int KST = D * 2 + 16;   // bytes per K row
-  static constexpr int VST = TK * 2 + 8;   // bytes per V^T row
-  static constexpr int K_BYTES = TK * KST;
-  static constexpr int V_BYTES = D * VST;
-  static constexpr int OST = D * 2 + 16;   // bytes per O staging row
-  static constexpr int TILE_BYTES = 2 * K_BYTES + 2 * V_BYTES;  // double-buffered K and V^T
-};
-
-// tile descriptor, word 0: level (2 bits) | masked (1) | nvalid 0..64 (7) | tile index inside the level (22)
-//                  word 1: offset of the level's block list (16) | number of blocks of the level (16)
-__device__ __forceinline__ u32x2 make_desc(int lv, bool masked, int nvalid, int lt, int ioff, int cnt) {
-  u32x2 d;
-  d[0] = (uint32_t)lv | ((uint32_t)masked << 2) | ((uint32_t)nvalid << 3) | ((uint32_t)lt << 10);
-  d[1] = (uint32_t)ioff | ((uint32_t)cnt << 16);
-  return d;
-}
-
-// Source row (in the level's own row numbering) of tile slot r, or -1 when the slot is empty.
-// The retained blocks of a level form one stream of cnt * 2^sbs_log2 pooled keys; tile lt covers
-// stream positions [64 lt, 64 lt + 64).
-__device__ __forceinline__ int slot_src(int lv, int lt, int r, int sbs_log2, int cnt, const uint16_t* ids, int L) {
-  const int g = (lt << 6) + r;
-  const int bi = g >> sbs_log2;
-  if (bi >= cnt) return -1;
-  const int src = ((int)ids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
-  return (lv == 0 && src >= L) ? -1 : src;
-}
-
-template <int D, int NW>
-#ifndef PSA_FWD_OCC
-#define PSA_FWD_OCC 2
-#endif
-__global__ __launch_bounds__(NW * 64, PSA_FWD_OCC) void psa_fwd_kernel(FwdParams p) {
-  // scalar copies of the arguments: lambdas below must not capture the argument struct itself
-  const auto P_B = p.B;
-  const auto P_Hkv = p.Hkv;
-  const auto P_L = p.L;
-  const auto P_bm = p.bm;
-  const auto P_bn_log2 = p.bn_log2;
-  const auto P_causal = p.causal;
-  const auto P_k = p.k;
-  const auto P_k_sb = p.k_sb;
-  const auto P_k_sh = p.k_sh;
-  const auto P_k_sl = p.k_sl;
-  const auto P_kp = p.kp;
-  const auto P_npad = p.npad;
-  const auto P_scale_log2 = p.scale_log2;
-  const auto P_v = p.v;
-  const auto P_v_sb = p.v_sb;
-  const auto P_v_sh = p.v_sh;
-  const auto P_v_sl = p.v_sl;
-  const auto P_vp = p.vp;
-  constexpr int NT = NW * 64;
-  constexpr int BM = NW * 32;
-  constexpr int CH = D / 8;           // 16-byte chunks per row
-  constexpr int UNITS = 16 * CH;      // (4 keys x 1 chunk) units per tile
-  constexpr int PER = (UNITS + NT - 1) / NT;
-  constexpr int KK = D / 16;          // MFMA k-steps for QK^T
-  constexpr int DB = D / 32;          // 32-row blocks of O^T
-  using SM = Smem<D>;
-  static_assert(BM * SM::OST <= SM::TILE_BYTES, "O staging must fit the tile buffers");
-
-  extern __shared__ __align__(16) unsigned char smem[];
-  auto Kbuf = [&](int i) __attribute__((always_inline)) -> unsigned char* { return smem + (i & 1) * SM::K_BYTES; };
-  auto Vbuf = [&](int i) __attribute__((always_inline)) -> unsigned char* { return smem + 2 * SM::K_BYTES + (i & 1) * SM::V_BYTES; };
-  u32x2* tdesc = (u32x2*)(smem + SM::TILE_BYTES);
-  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
-  __shared__ int s_cnt[4], s_ioff[4], s_toff[5];
-
-  // XCD-aware decode: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
-  // contiguous range of (b, h, q-block) so that one XCD's L2 sees few heads at a time.
-  const int bid = blockIdx.x;
-  // workgroup ids go round-robin over the 8 XCDs; slot s of XCD x works on row (s % chunk) of group 8*(s / chunk) + x
-  int logical = (((bid >> 3) / p.wg_chunk) * 8 + (bid & 7)) * p.wg_chunk + (bid >> 3) % p.wg_chunk;
-  if (p.order != nullptr) logical = p.order[logical];
-  if (logical < 0 || logical >= p.total_wg) return;
-  const int I = logical % p.Mq;
-  const int bh = logical / p.Mq;
-  const int h = bh % p.Hq, b = bh / p.Hq;
-  const int hk = h / (p.Hq / P_Hkv);
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, hh = lane >> 5;
-
-  // ---- 1. compact the map row into per-level lists ------------------------------------
-  int jmax = p.Nk;
-  if (P_causal) {
-    const int ce = (int)((((int64_t)(I + 1) * P_bm) + (1 << P_bn_log2) - 1) >> P_bn_log2);
-    jmax = ce < jmax ? ce : jmax;
-  }
-  if (wave == 0) {
-    int cnt[4] = {0, 0, 0, 0};
-    const int64_t mrow = ((int64_t)bh * p.Mq + I) * p.Nk;
-    if (p.map == nullptr) {
-      cnt[0] = jmax;
-      for (int j = lane; j < jmax; j += 64) ids[j] = (uint16_t)j;
-    } else {
-      for (int j0 = 0; j0 < jmax; j0 += 64) {
-        const int j = j0 + lane;
-        const int lvl = j < jmax ? load_map(p.map, mrow + j, p.map_elem) : 0;
-#pragma unroll
-        for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
-      }
-      int run[4];
-      run[0] = 0; run[1] = cnt[0]; run[2] = cnt[0] + cnt[1]; run[3] = cnt[0] + cnt[1] + cnt[2];
-      const uint64_t lt_mask = (1ull << lane) - 1ull;
-      for (int j0 = 0; j0 < jmax; j0 += 64) {
-        const int j = j0 + lane;
-        const int lvl = j < jmax ? load_map(p.map, mrow + j, p.map_elem) : 0;
-#pragma unroll
-        for (int lv = 0; lv < 4; ++lv) {
-          const uint64_t bal = __ballot(lvl == (1 << lv));
-          if (lvl == (1 << lv)) ids[run[lv] + __popcll(bal & lt_mask)] = (uint16_t)j;
-          run[lv] += __popcll(bal);
-        }
-      }
-    }
-    if (lane == 0) {
-      int io = 0, to = 0;
-#pragma unroll
-      for (int lv = 0; lv < 4; ++lv) {
-        const int c = lv == 0 ? cnt[0] : lv == 1 ? cnt[1] : lv == 2 ? cnt[2] : cnt[3];
-        const int sbs_log2 = P_bn_log2 - lv;
-        s_cnt[lv] = c;
-        s_ioff[lv] = io;
-        s_toff[lv] = to;
-        io += c;
-        to += sbs_log2 >= 6 ? (c << (sbs_log2 - 6)) : ((c << sbs_log2) + 63) >> 6;
-      }
-      s_toff[4] = to;
-    }
-  }
-
-  // ---- 2. Q fragments (B operand of S^T = K Q^T): lane holds Q[row l32][16*kk + 8*hh .. +8] ---
-  const int q_row0 = I * BM + wave * 32;
-  const int q_idx = q_row0 + l32;
-  bf16x8 qf[KK];
-  {
-    const int qr = q_idx < P_L ? q_idx : P_L - 1;
-    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
-  }
-  __syncthreads();
-
-  const int T = __builtin_amdgcn_readfirstlane(s_toff[4]);
-
-  // ---- 3. tile descriptors ------------------------------------------------------------------
-  for (int t = tid; t < T; t += NT) {
-    const int lv = (t >= s_toff[1]) + (t >= s_toff[2]) + (t >= s_toff[3]);
-    const int lt = t - s_toff[lv];
-    const int c_lv = s_cnt[lv];
-    const int io_lv = s_ioff[lv];
-    const int sbs_log2 = P_bn_log2 - lv;
-    // valid slots form a prefix of the tile: the level's stream ends, or (level 0) the sequence does
-    int nvalid = (c_lv << sbs_log2) - (lt << 6);
-    nvalid = nvalid < TK ? nvalid : TK;
-    const int last_blk = ids[io_lv + (((lt << 6) + nvalid - 1) >> sbs_log2)];
-    if (lv == 0) {
-      const int over = (((lt << 6) + nvalid - 1) & ((1 << sbs_log2) - 1)) + 1 - (P_L - (last_blk << sbs_log2));
-      if (over > 0) nvalid = nvalid - over > 0 ? nvalid - over : 0;
-    }
-    const bool diag = P_causal && ((((int64_t)last_blk + 1) << P_bn_log2) - 1 > (int64_t)I * P_bm);
-    tdesc[t] = make_desc(lv, diag || nvalid < TK, nvalid, lt, io_lv, c_lv);
-  }
-
-  // level bases: level 0 is K/V itself; pooled level lv >= 1 starts npad - (npad >> (lv-1)) rows into the
-  // pooled buffer (all batches and heads of a level are contiguous)
-  const bf16_t* kb0 = P_k + b * P_k_sb + hk * P_k_sh;
-  const bf16_t* vb0 = P_v + b * P_v_sb + hk * P_v_sh;
-  const int64_t BHkv = (int64_t)P_B * P_Hkv, bhk = (int64_t)b * P_Hkv + hk;
-
-  struct TileRef {
-    int lv, lt, cnt, sbs_log2;
-    const uint16_t* ids;
-    int64_t pool_off;
-  };
-  auto tile_ref = [&](int t) __attribute__((always_inline)) -> TileRef {
-    const u32x2 d = tdesc[t];
-    const uint32_t d0 = __builtin_amdgcn_readfirstlane(d[0]);
-    const uint32_t d1 = __builtin_amdgcn_readfirstlane(d[1]);
-    TileRef r;
-    r.lv = d0 & 3;
-    r.lt = d0 >> 10;
-    r.cnt = d1 >> 16;
-    r.ids = ids + (d1 & 0xffff);
-    r.sbs_log2 = P_bn_log2 - r.lv;
-    const int lm1 = r.lv > 0 ? r.lv - 1 : 0;
-    r.pool_off = (BHkv * (P_npad - (P_npad >> lm1)) + bhk * (P_npad >> r.lv)) * D;
-    return r;
-  };
-  // one (4 keys x 8 channels) unit per thread and PER
-  // Thread -> (key quad, 16-byte channel chunk) assignment.  K: neighbouring lanes walk along a row
-  // (whole 256-byte rows per 16 lanes).  V: neighbouring lanes walk along the key quads of one chunk,
-  // so that the transposed 8-byte LDS writes of 16 lanes fall into 16 different bank pairs.
-  auto unit_kq = [&](int u, bool vmap) __attribute__((always_inline)) { return vmap ? (u & 15) : (u / CH); };
-  auto unit_ch = [&](int u, bool vmap) __attribute__((always_inline)) { return vmap ? (u >> 4) : (u % CH); };
-  auto load_rows = [&](int t, const bf16_t* base0, int64_t str0, const bf16_t* pool, u32x4 (&reg)[PER][4], bool vmap) {
-    const TileRef r = tile_ref(t);
-    // uniform base pointer + 32-bit per-lane byte offset (a (b, h) slice is far below 4 GiB)
-    const char* base = (const char*)(r.lv == 0 ? base0 : pool + r.pool_off);
-    const uint32_t strb = r.lv == 0 ? (uint32_t)str0 * 2u : (uint32_t)(D * 2);
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = unit_kq(u, vmap) * 4, ch = unit_ch(u, vmap);
-      // 4 rows share a sub-block.  Empty slots load row 0 of the level (finite data): their logits are
-      // masked to -inf, so they contribute exactly 0.
-      const int src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
-      const int lim = r.lv == 0 ? P_L : 0x7fffffff;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int src = src0 + i;
-        src = (src0 >= 0 && src < lim) ? src : 0;
-        reg[u_][i] = *(const u32x4*)(base + ((uint32_t)src * strb + (uint32_t)(ch * 16)));
-      }
-    }
-  };
-  auto store_k = [&](unsigned char* Ks, const u32x4 (&reg)[PER][4]) {
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u / CH) * 4, ch = u % CH;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *(u32x4*)(Ks + (r0 + i) * SM::KST + ch * 16) = reg[u_][i];
-    }
-  };
-  auto store_vt = [&](unsigned char* Vt, const u32x4 (&reg)[PER][4]) {
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = unit_kq(u, true) * 4, ch = unit_ch(u, true);
-      // transpose 4 keys x 8 channels -> 8 channels x 4 keys
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        u32x2 e0, e1;
-        e0[0] = __builtin_amdgcn_perm(reg[u_][1][j], reg[u_][0][j], 0x05040100u);
-        e0[1] = __builtin_amdgcn_perm(reg[u_][3][j], reg[u_][2][j], 0x05040100u);
-        e1[0] = __builtin_amdgcn_perm(reg[u_][1][j], reg[u_][0][j], 0x07060302u);
-        e1[1] = __builtin_amdgcn_perm(reg[u_][3][j], reg[u_][2][j], 0x07060302u);
-        *(u32x2*)(Vt + (ch * 8 + 2 * j) * SM::VST + r0 * 2) = e0;
-        *(u32x2*)(Vt + (ch * 8 + 2 * j + 1) * SM::VST + r0 * 2) = e1;
-      }
-    }
-  };
-  // ---- 4. main loop -------------------------------------------------------------------------
-  f32x16 acc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  float m_run = -INFINITY;  // running reference max (log2 domain), same in both half-waves
-  float l_run = 0.f;        // this lane's partial row sum
-
-  if (T > 0) {
-    __syncthreads();  // tile descriptors visible
-    u32x4 kreg[PER][4], vreg[PER][4];
-    const int Tm1 = T - 1;
-    auto clampt = [&](int t) __attribute__((always_inline)) { return t < Tm1 ? t : Tm1; };
-    // prologue: tile 0 -> LDS buffers 0, tile 1 in flight
-    load_rows(0, kb0, P_k_sl, P_kp, kreg, false);
-    load_rows(0, vb0, P_v_sl, P_vp, vreg, true);
-    store_k(Kbuf(0), kreg);
-    store_vt(Vbuf(0), vreg);
-    load_rows(clampt(1), kb0, P_k_sl, P_kp, kreg, false);
-    load_rows(clampt(1), vb0, P_v_sl, P_vp, vreg, true);
-    __syncthreads();
-
-    for (int t = 0; t < T; ++t) {
-      // invariant: LDS buffers t&1 hold tile t; kreg/vreg hold tile t+1 (loads issued one step ago)
-      const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
-      const int lv = d & 3;
-      store_k(Kbuf(t + 1), kreg);
-      store_vt(Vbuf(t + 1), vreg);
-      load_rows(clampt(t + 2), kb0, P_k_sl, P_kp, kreg, false);
-      load_rows(clampt(t + 2), vb0, P_v_sl, P_vp, vreg, true);
-
-      // S^T = K Q^T: two independent 32-key accumulation chains; LDS operands are fetched one k-step ahead
-      const unsigned char* Ks = Kbuf(t) + l32 * SM::KST + hh * 16;
-      f32x16 s_cur[2];
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_cur[c][i] = 0.f;
-      {
-        bf16x8 a0 = *(const bf16x8*)(Ks), a1 = *(const bf16x8*)(Ks + 32 * SM::KST);
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          bf16x8 n0 = a0, n1 = a1;
-          if (kk + 1 < KK) {
-            n0 = *(const bf16x8*)(Ks + (kk + 1) * 32);
-            n1 = *(const bf16x8*)(Ks + 32 * SM::KST + (kk + 1) * 32);
-          }
-          s_cur[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s_cur[0], 0, 0, 0);
-          s_cur[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s_cur[1], 0, 0, 0);
-          a0 = n0;
-          a1 = n1;
-        }
-      }
-
-      if (d & 4) {  // partly empty tile and/or causal diagonal: mask individual keys
-        const TileRef r = tile_ref(t);
-        const int nvalid = (int)((d >> 3) & 127);
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int r0 = c * 32 + g * 8 + hh * 4;
-            int src0 = -1;
-            if (r0 < nvalid) src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, P_L);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const bool in_tile = src0 >= 0 && (r0 + e) < nvalid;
-              // causal: a pooled key is visible once its last constituent token is
-              const bool visible = !P_causal || ((((int64_t)(src0 + e) + 1) << lv) - 1 <= (int64_t)q_idx);
-              const float sv = s_cur[c][g * 4 + e];
-              s_cur[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
-            }
-          }
-      }
-
-      // online softmax of tile t (per query column = per lane, both half-waves)
-      float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
-#pragma unroll
-      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s_cur[0][i], s_cur[1][i]));
-      mx = half_wave_max(mx);
-      const float bias = (float)lv;
-      const float m_cand = __builtin_fmaf(mx, P_scale_log2, bias);
-      // raise the reference max only when it lags by more than the threshold (or is still -inf)
-      float m_new = (m_cand - m_run > LAZY_THRESHOLD) ? m_cand : m_run;
-      m_new = (m_run == -INFINITY) ? m_cand : m_new;
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // rows that still see no key
-      const float alpha = fast_exp2(m_run - m_use);
-      const float nb = bias - m_use;
-      float lsum0 = 0.f, lsum1 = 0.f;
-      uint32_t pk[2][8];
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float p0 = fast_exp2(__builtin_fmaf(s_cur[c][i], P_scale_log2, nb));
-          const float p1 = fast_exp2(__builtin_fmaf(s_cur[c][i + 1], P_scale_log2, nb));
-          lsum0 += p0;
-          lsum1 += p1;
-          pk[c][i >> 1] = pack_bf16x2(p0, p1);
-        }
-      }
-      l_run = l_run * alpha + (lsum0 + lsum1);
-      m_run = m_new;
-
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
-      }
-
-      // O^T += V^T P^T : per 16-key group g, A = V^T[32 d][16 keys], B = P^T[16 keys][32 q];
-      // the V^T operands of the next group are fetched while the current group's MFMAs issue
-      const unsigned char* Vt = Vbuf(t) + l32 * SM::VST + hh * 8;
-      u32x2 vlo[DB], vhi[DB];
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        vlo[db] = *(const u32x2*)(Vt + db * 32 * SM::VST);
-        vhi[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + 16);
-      }
-#pragma unroll
-      for (int cg = 0; cg < 4; ++cg) {
-        const int c = cg >> 1, g = cg & 1;
-        u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
-        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
-        u32x2 nlo[DB], nhi[DB];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          nlo[db] = vlo[db];
-          nhi[db] = vhi[db];
-          if (cg + 1 < 4) {
-            nlo[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + (cg + 1) * 32);
-            nhi[db] = *(const u32x2*)(Vt + db * 32 * SM::VST + (cg + 1) * 32 + 16);
-          }
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          u32x4 aw = {vlo[db][0], vlo[db][1], vhi[db][0], vhi[db][1]};
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          vlo[db] = nlo[db];
-          vhi[db] = nhi[db];
-        }
-      }
-      __syncthreads();
-    }
-  }
-
-  // ---- 5. epilogue --------------------------------------------------------------------------
-  float l_tot = half_wave_sum(l_run);
-  const float l_safe = fmaxf(l_tot, 1e-8f);
-  const float inv = 1.0f / l_safe;
-  if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
-    // natural-log domain: m*ln2 + ln(max(l, 1e-8))
-    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
-  }
-  __syncthreads();  // everyone is done with the last K/V tile
-  unsigned char* Os = smem;
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      u32x2 w;
-      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
-      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
-      *(u32x2*)(Os + (wave * 32 + l32) * SM::OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
-    }
-  __syncthreads();
-  bf16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
-  for (int u = tid; u < BM * CH; u += NT) {
-    const int r = u / CH, ch = u % CH;
-    const int row = I * BM + r;
-    if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * SM::OST + ch * 16);
-  }
-}
-
-// =========================================================================================================
-// Head dim 128: tiles go from global memory straight into LDS (no register staging), V is read back with
-// the transposing LDS load, and the exponentials of one tile overlap the QK^T MFMAs of the next.
-//
-//  * K and V tiles are both kept row-major in LDS, double buffered.  One global_load_lds_dwordx4 moves 4
-//    rows of 256 bytes (64 lanes x 16 bytes land at consecutive LDS addresses); the 16 four-row blocks of
-//    a tile are F_ISTR = 1024 + 64 bytes apart, and row q of a block stores its 16-byte chunks
-//    XOR-swizzled: chunk c sits at position c ^ q.  The swizzle is applied on the global side (a lane
-//    fetches the chunk that belongs at its LDS position), so it costs nothing.  Padding and swizzle together
-//    make the 128-bit K reads and the transposing V reads bank-conflict free, and both only touch the low
-//    bits of the chunk index, so every operand address is lane base + immediate.
-//  * Inside each group of 16 rows the rows are stored 4x4-transposed (block n, row q holds tile slot
-//    4q + n): the 4 rows a lane fetches are then 4 CONSECUTIVE tile slots, which always belong to one
-//    kv-block, so one block-list lookup per lane and tile serves K and V.
-//  * ds_read_b64_tr_b16 hands every lane 4 keys of one channel from row-major V: exactly the A operand
-//    of O^T += V^T P^T, in the key order that the S^T accumulator layout gives P^T.
-//  * The tile loop is unrolled by two so that the LDS buffer offsets are immediates.
-constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the 4-row blocks of a tile
-constexpr int F_TILE = psa_tiles::LT_TILE;  // bytes of one K or V tile (D = 128)
+constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the blocks of a tile
 
 
 #define TILE_SYNC()                         \
@@ -508,9 +62,11 @@ constexpr int F_TILE = psa_tiles::LT_TILE;  // bytes of one K or V tile (D = 128
     __syncthreads();                        \
   } while (0)
 
-template <int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
-  constexpr int D = 128, NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
+template <int D, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
+  using G = psa_tiles::LtGeom<D>;
+  constexpr int F_TILE = G::TILE;  // bytes of one K or V tile
+  constexpr int NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
   constexpr int G16 = 4 / NW;  // 16-row groups of a tile fetched by one wave
   constexpr int OST = D * 2 + 16;
   static_assert(NW == 4 || NW == 2 || NW == 1, "1, 2 or 4 waves");
@@ -565,19 +121,19 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
 
   // ---- lane-invariant addressing (tile layout: psa_tiles.h) -------------------------------------------
-  const uint32_t f_chunk = psa_tiles::lt_fetch_chunk(lane);
+  const uint32_t f_chunk = psa_tiles::lt_fetch_chunk<D>(lane);
   uint32_t k_off[2], v_off[2];
-  psa_tiles::lt_row_operand(l32, hh, k_off);  // K rows l32 (+32): k_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
-  psa_tiles::lt_tr_operand(lane, v_off);      // V^T: v_off[s] + 64 * db + 4 * F_ISTR * cg
+  psa_tiles::lt_row_operand<D>(l32, hh, k_off);  // K rows l32 (+32): k_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
+  psa_tiles::lt_tr_operand<D>(lane, v_off);      // V^T: v_off[s] + 64 * db + 4 * F_ISTR * cg
 
   psa_tiles::KvSource kvs;
   kvs.k0 = kb0; kvs.v0 = vb0; kvs.kp = (const char*)P_kp; kvs.vp = (const char*)P_vp;
   kvs.k_strb = P_k_strb; kvs.v_strb = P_v_strb;
   kvs.BHkv = BHkv; kvs.bhk = bhk; kvs.npad = P_npad; kvs.bn_log2 = P_bn_log2; kvs.L = P_L;
   using TileSrc = psa_tiles::TileSrc<G16>;
-  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) { psa_tiles::lt_tile_src<G16>(kvs, tdesc, ids, t, wave, lane, a); };
+  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) { psa_tiles::lt_tile_src<D, G16>(kvs, tdesc, ids, t, wave, lane, a); };
   auto issue_rows = [&](const char* base, uint32_t str, int lim, const int (&src0)[G16], int lds_byte) __attribute__((always_inline)) {
-    psa_tiles::lt_issue_rows<G16>(smem + lds_byte, base, str, lim, src0, wave, f_chunk);
+    psa_tiles::lt_issue_rows<D, G16>(smem + lds_byte, base, str, lim, src0, wave, f_chunk);
   };
 
   f32x16 acc[DB];
@@ -660,13 +216,13 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s2[c][i] = 0.f;
-    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 8 * F_ISTR);
+    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + G::HALF);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       bf16x8 n0 = a0, n1 = a1;
       if (kk + 1 < KK) {
         n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
-        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + 8 * F_ISTR);
+        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + G::HALF);
       }
       s2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s2[0], 0, 0, 0);
       s2[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s2[1], 0, 0, 0);
@@ -678,12 +234,12 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
   // transposing reads), B = P^T.  8 MFMAs on 4 independent accumulators.
   auto pv_half = [&](auto vb_c, int hf, const uint32_t* pk8) __attribute__((always_inline)) {
     constexpr int VB = decltype(vb_c)::value;
-    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + VB) * F_TILE + hf * (8 * F_ISTR);
-    // operand of MFMA step st = 4*g + db; reads run AHEAD steps in front of the MFMAs
+    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem) + (2 + VB) * F_TILE + hf * G::HALF;
+    // operand of MFMA step st = DB*g + db; reads run AHEAD steps in front of the MFMAs
     constexpr int AHEAD = 2, STEPS = 2 * DB;
     auto vread = [&](int st, int s) __attribute__((always_inline)) {
       return __builtin_bit_cast(
-          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[s] + (st & 3) * 64 + (st >> 2) * (4 * F_ISTR))));
+          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[s] + (st % DB) * 64 + (st / DB) * G::GROUP)));
     };
     u32x2 vlo[STEPS], vhi[STEPS];  // fully unrolled: every element is a short-lived register value
 #pragma unroll
@@ -693,7 +249,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_d128_kernel(FwdParams p) {
     }
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
-      const int g = st >> 2, db = st & 3;
+      const int g = st / DB, db = st % DB;
       if (st + AHEAD < STEPS) {
         vlo[st + AHEAD] = vread(st + AHEAD, 0);
         vhi[st + AHEAD] = vread(st + AHEAD, 1);
@@ -856,24 +412,11 @@ __global__ __launch_bounds__(256) void psa_fwd_sort_kernel(const int32_t* cost, 
 
 template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
-  using SM = Smem<D>;
-  size_t shmem = (size_t)SM::TILE_BYTES + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
+  size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
   if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-  if (shmem > 48 * 1024) {
-    if (hipFuncSetAttribute((const void*)psa_fwd_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-      return PSA_ERR_LAUNCH;
-  }
-  hipLaunchKernelGGL((psa_fwd_kernel<D, NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
-  return PSA_OK;
-}
-
-template <int NW>
-int launch_fwd_d128(const FwdParams& p, int Nk, hipStream_t stream) {
-  size_t shmem = (size_t)4 * F_TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
-  if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-  if (hipFuncSetAttribute((const void*)psa_fwd_d128_kernel<NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+  if (hipFuncSetAttribute((const void*)psa_fwd_lds_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
     return PSA_ERR_LAUNCH;
-  hipLaunchKernelGGL((psa_fwd_d128_kernel<NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
+  hipLaunchKernelGGL((psa_fwd_lds_kernel<D, NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
   return PSA_OK;
 }
 
@@ -947,8 +490,8 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     p.order = order;
   }
   int rc;
-  if (D == 128 && block_m == 128) rc = launch_fwd_d128<4>(p, Nk, (hipStream_t)stream);
-  else if (D == 128) rc = launch_fwd_d128<2>(p, Nk, (hipStream_t)stream);
+  if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
+  else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);
   else if (block_m == 128) rc = launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
   else rc = launch_fwd<64, 2>(p, Nk, (hipStream_t)stream);
   PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");

@@ -165,46 +165,83 @@ __device__ __forceinline__ int64_t pool_row_offset(int lv, int64_t BHkv, int64_t
 }
 
 // ------------------------------------------------------------------------------------------------------
-// LDS tile layout of the head-dim-128 kernels (64 rows x 256 bytes, filled by global_load_lds_dwordx4).
-//   * a tile is 16 blocks of 4 rows, blocks LT_ISTR = 1024 + 64 bytes apart (one copy instruction per block:
-//     64 lanes x 16 bytes land at consecutive LDS addresses);
-//   * row q of a block stores its 16-byte chunks XOR-swizzled: chunk c sits at position c ^ q (applied on the
-//     global side: a lane fetches the chunk that belongs at its LDS position);
-//   * inside each group of 16 rows the rows are stored 4x4-transposed: block n, row q holds tile row 4q + n,
-//     so the 4 rows a lane fetches are 4 CONSECUTIVE tile rows.
+// LDS tile layout of the kernels that copy tiles with global_load_lds_dwordx4: 64 rows of D bf16 values.
+//   * One copy instruction moves 1024 bytes (64 lanes x 16 bytes land at consecutive LDS addresses), i.e. a
+//     BLOCK of RPB = 512 / D rows (4 rows of 256 bytes for D = 128, 8 rows of 128 bytes for D = 64); the blocks
+//     of a tile are LT_ISTR = 1024 + 64 bytes apart.
+//   * Row r of a block stores its 16-byte chunks XOR-swizzled: chunk c sits at position c ^ (r * RPB / 16)...
+//     in short c ^ r for D = 128 and c ^ (r >> 1) for D = 64 (applied on the global side: a lane fetches the
+//     chunk that belongs at its LDS position).
+//   * Inside each group of 16 tile rows the rows are stored transposed (block n, row r holds tile row
+//     RPL * r + n, RPL = 16 / RPB blocks per group), so the RPL rows a lane fetches are CONSECUTIVE tile rows.
 // Padding and swizzle make the 128-bit row reads and the transposing reads bank-conflict free, and both only
-// touch the low bits of the chunk index, so every operand address is lane base + immediate.
+// touch the low two bits of the chunk index, so every operand address is lane base + immediate.
 // ------------------------------------------------------------------------------------------------------
 constexpr int LT_ISTR = 1024 + 64;
-constexpr int LT_TILE = 16 * LT_ISTR;
+template <int D>
+struct LtGeom {
+  static constexpr int CH = D / 8;          // 16-byte chunks per row
+  static constexpr int RPB = 64 / CH;       // rows per block (per copy instruction)
+  static constexpr int RPL = 16 / RPB;      // blocks per 16-row group = consecutive tile rows per lane
+  static constexpr int BLOCKS = 64 / RPB;   // blocks per tile
+  static constexpr int TILE = BLOCKS * LT_ISTR;
+  static constexpr int SW_SHIFT = RPB == 4 ? 0 : 1;  // swizzle key of block row r: r >> SW_SHIFT (0..3)
+  static constexpr int HALF = (32 / RPB) * LT_ISTR;  // byte distance of tile rows r and r + 32
+  static constexpr int GROUP = RPL * LT_ISTR;        // byte distance of consecutive 16-row groups
+};
+constexpr int LT_TILE = LtGeom<128>::TILE;
 
 #define PSA_LDS(T) __attribute__((address_space(3))) T*
 
-// copy side: byte offset of the chunk a lane fetches, and the first of its 4 tile rows inside a 16-row group
-__device__ __forceinline__ uint32_t lt_fetch_chunk(int lane) { return (uint32_t)(((lane & 15) ^ (lane >> 4)) * 16); }
-__device__ __forceinline__ int lt_fetch_row(int lane) { return (lane >> 4) * 4; }
+// copy side: byte offset of the chunk a lane fetches, and the first of its RPL tile rows inside a 16-row group
+template <int D>
+__device__ __forceinline__ uint32_t lt_fetch_chunk(int lane) {
+  using G = LtGeom<D>;
+  const int r = lane / G::CH, pos = lane % G::CH;
+  return (uint32_t)((pos ^ (r >> G::SW_SHIFT)) * 16);
+}
+template <int D>
+__device__ __forceinline__ int lt_fetch_row(int lane) {
+  using G = LtGeom<D>;
+  return (lane / G::CH) * G::RPL;
+}
+
+// physical position of tile row `row`: block index and row inside the block
+template <int D>
+__device__ __forceinline__ void lt_place(int row, int& block, int& r) {
+  using G = LtGeom<D>;
+  const int in_group = row & 15;
+  block = (row >> 4) * G::RPL + in_group % G::RPL;
+  r = in_group / G::RPL;
+}
 
 // MFMA row operand (A: 32 tile rows x 16 channels) of k-step kk for tile row `row`, hh = lane / 32:
 // off[kk & 1] + 64 * (kk >> 1)
+template <int D>
 __device__ __forceinline__ void lt_row_operand(int row, int hh, uint32_t (&off)[2]) {
-  const int q = (row >> 2) & 3;
-  const int base = (4 * (row >> 4) + (row & 3)) * LT_ISTR + q * 256;
-  off[0] = (uint32_t)(base + ((hh ^ q) * 16));
-  off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
+  using G = LtGeom<D>;
+  int block, r;
+  lt_place<D>(row, block, r);
+  const int base = block * LT_ISTR + r * (D * 2), f = r >> G::SW_SHIFT;
+  off[0] = (uint32_t)(base + ((hh ^ f) * 16));
+  off[1] = (uint32_t)(base + (((2 + hh) ^ f) * 16));
 }
 
 // MFMA transposed operand (A: 32 channels x 16 tile rows) through ds_read_b64_tr_b16.  Inside a block of 16
 // lanes, lane i supplies the address of 4 channels (4*(i%4)..) of row i/4 and receives channel i of the
-// block's 4 rows.  Lane block bl covers channels 32*db + 16*(bl&1).. and rows 16*grp + 8*s + 4*(bl>>1)..
-// (s = first / second half of the operand): off[s] + 64 * db + 4 * LT_ISTR * grp.  The row order inside the
+// block's 4 rows.  Lane block bl covers channels 32*db + 16*(bl&1).. and tile rows 16*grp + 8*s + 4*(bl>>1)..
+// (s = first / second half of the operand): off[s] + 64 * db + GROUP * grp.  The row order inside the
 // operand equals the order in which the 32x32 MFMA accumulator layout hands 8 consecutive registers to a lane.
+template <int D>
 __device__ __forceinline__ void lt_tr_operand(int lane, uint32_t (&off)[2]) {
+  using G = LtGeom<D>;
   const int i16 = lane & 15, bl = lane >> 4;
-  const int n = i16 >> 2, cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
+  const int cl = 2 * (bl & 1) + ((i16 & 3) >> 1), hb = i16 & 1;
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    const int qq = 2 * s + (bl >> 1);
-    off[s] = (uint32_t)(n * LT_ISTR + qq * 256 + ((cl ^ qq) * 16) + hb * 8);
+    int block, r;
+    lt_place<D>(8 * s + 4 * (bl >> 1) + (i16 >> 2), block, r);
+    off[s] = (uint32_t)(block * LT_ISTR + r * (D * 2) + ((cl ^ (r >> G::SW_SHIFT)) * 16) + hb * 8);
   }
 }
 
@@ -223,10 +260,10 @@ struct TileSrc {
   const char *kbase, *vbase;
   uint32_t kstr, vstr;
   int lim;        // last valid row when the tile may run past the sequence end, else INT_MAX
-  int src0[G16];  // first of the lane's 4 consecutive source rows, per group
+  int src0[G16];  // first of the lane's consecutive source rows, per group
 };
 
-template <int G16>
+template <int D, int G16>
 __device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tdesc, const uint16_t* ids, int t, int wave, int lane,
                                             TileSrc<G16>& a) {
   const u32x2 dd = tdesc[t];
@@ -237,38 +274,39 @@ __device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tde
   const uint16_t* lids = ids + (d1 & 0xffff);
   const int sbs_log2 = kv.bn_log2 - lv;
   const int lm1 = lv > 0 ? lv - 1 : 0;
-  const int64_t pool_off = (kv.BHkv * (kv.npad - (kv.npad >> lm1)) + kv.bhk * (kv.npad >> lv)) * 256;
+  const int64_t pool_off = (kv.BHkv * (kv.npad - (kv.npad >> lm1)) + kv.bhk * (kv.npad >> lv)) * (D * 2);
   a.kbase = lv == 0 ? kv.k0 : kv.kp + pool_off;
   a.vbase = lv == 0 ? kv.v0 : kv.vp + pool_off;
-  a.kstr = lv == 0 ? kv.k_strb : 256u;
-  a.vstr = lv == 0 ? kv.v_strb : 256u;
+  a.kstr = lv == 0 ? kv.k_strb : (uint32_t)(D * 2);
+  a.vstr = lv == 0 ? kv.v_strb : (uint32_t)(D * 2);
   const bool ragged = nvalid < TK;  // some slots are empty: clamp them onto real rows (their logits are masked)
   a.lim = (ragged && lv == 0) ? kv.L - 1 : 0x7fffffff;
 #pragma unroll
   for (int gi = 0; gi < G16; ++gi) {
-    const int g = (lt << 6) + (wave * G16 + gi) * 16 + lt_fetch_row(lane);
+    const int g = (lt << 6) + (wave * G16 + gi) * 16 + lt_fetch_row<D>(lane);
     int bi = g >> sbs_log2;
     if (ragged) bi = bi < cnt - 1 ? bi : cnt - 1;
     a.src0[gi] = ((int)lids[bi] << sbs_log2) + (g & ((1 << sbs_log2) - 1));
   }
 }
 
-// Copies this wave's groups of one tile: 4 rows per instruction go to block 4*g16 + n of the tile at `dst`.
-template <int G16>
+// Copies this wave's groups of one tile: one block per instruction goes to block RPL*g16 + n of the tile at `dst`.
+template <int D, int G16>
 __device__ __forceinline__ void lt_issue_rows(unsigned char* dst, const char* base, uint32_t str, int lim, const int (&src0)[G16],
                                               int wave, uint32_t f_chunk) {
+  using G = LtGeom<D>;
 #pragma unroll
   for (int gi = 0; gi < G16; ++gi) {
-    const int blk = (wave * G16 + gi) * 4;
+    const int blk = (wave * G16 + gi) * G::RPL;
     if (lim == 0x7fffffff) {
       // the usual case: the uniform base pointer steps from row to row, the lane offset stays
       const uint32_t off = (uint32_t)src0[gi] * str + f_chunk;
 #pragma unroll
-      for (int n = 0; n < 4; ++n)
+      for (int n = 0; n < G::RPL; ++n)
         __builtin_amdgcn_global_load_lds(base + (uint64_t)(n * str) + off, (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
     } else {
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
+      for (int n = 0; n < G::RPL; ++n) {
         const int src = src0[gi] + n < lim ? src0[gi] + n : lim;
         __builtin_amdgcn_global_load_lds(base + ((uint32_t)src * str + f_chunk), (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
       }
