@@ -6,14 +6,17 @@
 //
 // Kernel 1 (MFMA-bound, 2*Ms*Ns*D flops): a dense bf16 contraction of the sampled query rows with the
 // sampled key rows, both gathered straight from the un-sampled Q / K through the per-head offset
-// tables.  One workgroup = NW waves x 32 sampled query rows; the waves share K tiles of 64 sampled
-// keys, double-buffered in LDS (one barrier per tile, global loads two tiles ahead).  As in the
-// forward kernel the transposed product S^T = K Q^T is computed, so a lane holds 16 keys of one query
-// row and a key-group maximum is an in-lane reduction plus one half-wave exchange.  The group maxima
-// go to an fp32 workspace laid out [key group][query row], i.e. 128-byte coalesced stores.
+// tables.  One workgroup = 4 waves x 64 sampled query rows (two B-operand sets per wave share every K
+// operand read from LDS); the waves share K tiles of 64 sampled keys, copied by global_load_lds into
+// double-buffered LDS (one barrier per tile).  The key range is cut into 1, 2 or 4 shares (grid z) so that
+// the launch fills the chip; the row maxima of the shares are combined by kernel 2.  As in the forward
+// kernel the transposed product S^T = K Q^T is computed, so a lane holds 16 keys of one query row and a
+// key-group maximum is an in-lane v_max3 chain plus one half-wave exchange.  The group maxima go to an
+// fp32 workspace laid out [key group][query row] (128-byte coalesced stores, issued one tile late).
 // Kernel 2 (HBM-bound, reads the workspace once): per (query group, key group) the maximum over the
 // group's rows of R - m, exp2, row sum in a fixed order, normalisation.
 #include "psa_common.h"
+#include "psa_tiles.h"
 
 namespace {
 
@@ -43,161 +46,17 @@ __device__ __forceinline__ int sampled_src(int r, int n_real, int keep_log2, int
   return src < L ? src : L - 1;
 }
 
-template <int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_est_gemm_kernel(EstParams p) {
-  constexpr int NT = NW * 64;
-  constexpr int CH = D / 8;
-  constexpr int UNITS = 16 * CH;
-  constexpr int PER = (UNITS + NT - 1) / NT;
-  constexpr int KK = D / 16;
-  constexpr int KST = D * 2 + 16;
-  constexpr int K_BYTES = TK * KST;
-
-  __shared__ __align__(16) unsigned char smem[2 * K_BYTES];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, hh = lane >> 5;
-  const int bh = blockIdx.y;
-  const int h = bh % p.Hq, b = bh / p.Hq;
-  const int hk = h / (p.Hq / p.Hkv);
-  const int keep_m = 1 << p.keep_m_log2, keep_n = 1 << p.keep_n_log2;
-
-  // Q fragments
-  const int row0 = blockIdx.x * (NW * 32) + wave * 32;
-  bf16x8 qf[KK];
-  {
-    const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * keep_m : nullptr;
-    const int src = sampled_src(row0 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
-    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
-  }
-
-  const char* kb = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
-  const uint32_t kstrb = (uint32_t)p.k_sl * 2u;
-  const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * keep_n : nullptr;
-  // a thread always handles the same in-group positions: tiles are 64 keys and keep_n divides 64
-  int my_off[PER][4];
-#pragma unroll
-  for (int u_ = 0; u_ < PER; ++u_) {
-    const int u = tid + u_ * NT;
-    const int r0 = (u / CH) * 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = (r0 + i) & (keep_n - 1);
-      my_off[u_][i] = ok ? ok[e] : e;
-    }
-  }
-  const int Ns = p.Ns, Lk = p.Lk, bn = p.bn, kn_log2 = p.keep_n_log2;
-  u32x4 kreg[PER][4];
-  auto load_tile = [&](int t) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u / CH) * 4, ch = u % CH;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int r = t * TK + r0 + i;
-        int src;
-        if (r < Ns) {
-          src = (r >> kn_log2) * bn + my_off[u_][i];
-        } else {  // padding keys replicate the last sampled key
-          r = Ns - 1;
-          src = (r >> kn_log2) * bn + (ok ? ok[r & ((1 << kn_log2) - 1)] : (r & ((1 << kn_log2) - 1)));
-        }
-        src = src < Lk ? src : Lk - 1;
-        kreg[u_][i] = *(const u32x4*)(kb + ((uint32_t)src * kstrb + (uint32_t)(ch * 16)));
-      }
-    }
-  };
-  auto store_tile = [&](unsigned char* Ks) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u / CH) * 4, ch = u % CH;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *(u32x4*)(Ks + (r0 + i) * KST + ch * 16) = kreg[u_][i];
-    }
-  };
-
-  const int T = p.Ns_pad / TK;
-  const int gpc_log2 = 5 - p.keep_n_log2;  // key groups per 32-key chunk (1, 2 or 4)
-  float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + row0 + l32;
-  const int64_t rts = p.Ms_pad;
-  float m_run = -INFINITY;
-  const float qk_scale = p.qk_scale;
-
-  load_tile(0);
-  store_tile(smem);
-  load_tile(T > 1 ? 1 : 0);
-  __syncthreads();
-  for (int t = 0; t < T; ++t) {
-    // invariant: buffer t&1 holds tile t; kreg holds tile t+1 (in flight)
-    store_tile(smem + ((t + 1) & 1) * K_BYTES);
-    load_tile(t + 2 < T ? t + 2 : T - 1);
-    const unsigned char* Ks = smem + (t & 1) * K_BYTES;
-    f32x16 s[2];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const bf16x8 a = *(const bf16x8*)(Ks + (c * 32 + l32) * KST + hh * 16 + kk * 32);
-        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s[c], 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      // register i holds key (i/4)*8 + hh*4 + i%4 of this chunk: 8-key octets are registers 4o..4o+3
-      float o4[4];
-#pragma unroll
-      for (int o = 0; o < 4; ++o) o4[o] = fmaxf(fmaxf(s[c][4 * o], s[c][4 * o + 1]), fmaxf(s[c][4 * o + 2], s[c][4 * o + 3]));
-      const int jbase = (t * 2 + c) << gpc_log2;
-      if (gpc_log2 == 0) {
-        float v = fmaxf(fmaxf(o4[0], o4[1]), fmaxf(o4[2], o4[3]));
-        v = half_wave_max(v) * qk_scale;
-        m_run = fmaxf(m_run, v);
-        if (hh == 0) rt[(int64_t)jbase * rts] = v;
-      } else if (gpc_log2 == 1) {
-        float v0 = fmaxf(o4[0], o4[1]), v1 = fmaxf(o4[2], o4[3]);
-        v0 = half_wave_max(v0) * qk_scale;
-        v1 = half_wave_max(v1) * qk_scale;
-        m_run = fmaxf(m_run, fmaxf(v0, v1));
-        rt[(int64_t)(jbase + hh) * rts] = hh ? v1 : v0;
-      } else {
-#pragma unroll
-        for (int o = 0; o < 4; ++o) {
-          const float v = half_wave_max(o4[o]) * qk_scale;
-          m_run = fmaxf(m_run, v);
-          if ((o & 1) == hh) rt[(int64_t)(jbase + o) * rts] = v;
-        }
-      }
-    }
-    __syncthreads();
-  }
-  if (hh == 0) p.mrow[(int64_t)bh * p.ksplit * p.Ms_pad + row0 + l32] = m_run;
-}
-
-// Head dim 128: 64 sampled query rows per wave (two B-operand sets share every K operand fetched from LDS)
-// and K tiles copied from global memory straight into LDS, double buffered.
-//
-// LDS tile layout (shared with the attention forward kernel): a tile is 16 blocks of 4 rows x 256 bytes, blocks
-// E_ISTR = 1024 + 64 bytes apart; block n, row q of a 16-row group holds tile slot 4q + n, with its 16-byte
-// chunks XOR-swizzled by q.  One global_load_lds_dwordx4 fills one block; the 128-bit operand reads are bank
-// conflict free and their addresses are lane base + immediate.
-constexpr int E_ISTR = 1024 + 64;
-constexpr int E_TILE = 16 * E_ISTR;
+// 64 sampled query rows per wave (two B-operand sets share every K operand fetched from LDS) and K tiles
+// copied from global memory straight into LDS, double buffered, in the padded + swizzled tile layout of
+// psa_tiles.h (shared with the attention kernels): the 128-bit operand reads are bank-conflict free and their
+// addresses are lane base + immediate.
 constexpr int E_STAGES = 2;
 
-#define PSA_LDS(T) __attribute__((address_space(3))) T*
-
-__global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
-  constexpr int D = 128, KK = D / 16, RS = 2;  // RS sets of 32 query rows per wave
+template <int D>
+__global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
+  using G = psa_tiles::LtGeom<D>;
+  constexpr int KK = D / 16, RS = 2;  // RS sets of 32 query rows per wave
+  constexpr int E_TILE = G::TILE, E_ISTR = psa_tiles::LT_ISTR, RPL = G::RPL;
   __shared__ __align__(16) unsigned char smem[E_STAGES * E_TILE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -226,14 +85,12 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
   const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * keep_n : nullptr;
   const int Ns = p.Ns, Lk = p.Lk, bn = p.bn, kn_log2 = p.keep_n_log2;
 
-  // fetch: wave w copies the 16-row group w of a tile; lane (q = lane/16, pos = lane%16) of block n writes
-  // row q of that block at position pos, i.e. tile slot 16w + 4q + n, chunk pos ^ q
-  const int fq = lane >> 4;
-  const uint32_t f_chunk = (uint32_t)(((lane & 15) ^ fq) * 16);
-  const int slot0 = wave * 16 + fq * 4;  // first of this lane's 4 consecutive tile slots (inside one key group)
-  int my_off[4];
+  // fetch: wave w copies the 16-row group w of a tile, one block per instruction
+  const uint32_t f_chunk = psa_tiles::lt_fetch_chunk<D>(lane);
+  const int slot0 = wave * 16 + psa_tiles::lt_fetch_row<D>(lane);  // first of this lane's consecutive tile slots
+  int my_off[RPL];
 #pragma unroll
-  for (int n = 0; n < 4; ++n) {
+  for (int n = 0; n < RPL; ++n) {
     const int e = (slot0 + n) & (keep_n - 1);
     my_off[n] = ok ? ok[e] : e;
   }
@@ -242,7 +99,7 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
     const bool inside = (t + 1) * TK <= Ns && ((((t + 1) * TK - 1) >> kn_log2) + 1) * bn <= Lk;  // uniform
     const int grp_row = (r0 >> kn_log2) * bn;
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
+    for (int n = 0; n < RPL; ++n) {
       int src = grp_row + my_off[n];
       if (!inside) {
         // padding keys replicate the last sampled key; rows past the sequence end clamp to its last row
@@ -255,18 +112,12 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
         src = src < Lk ? src : Lk - 1;
       }
       __builtin_amdgcn_global_load_lds(kb + ((uint32_t)src * kstrb + f_chunk),
-                                       (PSA_LDS(void))(smem + stage * E_TILE + (wave * 4 + n) * E_ISTR), 16, 0, 0);
+                                       (PSA_LDS(void))(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR), 16, 0, 0);
     }
   };
-  // K operand of k-step kk: tile slot l32 (+32) = block 4*(l32>>4) + (l32&3), row (l32>>2)&3, chunk 2kk + hh
-  // -> k_off[kk & 1] + 64 * (kk >> 1)   (+ 8 blocks for the second 32 keys)
+  // K operand of k-step kk for tile slots l32 and l32 + 32: k_off[kk & 1] + 64 * (kk >> 1) (+ G::HALF)
   uint32_t k_off[2];
-  {
-    const int q = (l32 >> 2) & 3;
-    const int base = (4 * (l32 >> 4) + (l32 & 3)) * E_ISTR + q * 256;
-    k_off[0] = (uint32_t)(base + ((hh ^ q) * 16));
-    k_off[1] = (uint32_t)(base + (((2 + hh) ^ q) * 16));
-  }
+  psa_tiles::lt_row_operand<D>(l32, hh, k_off);
 
   const int T = p.Ns_pad / TK;
   const int gpc_log2 = 5 - p.keep_n_log2;  // key groups per 32-key chunk (1, 2 or 4)
@@ -318,13 +169,13 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm128_kernel(EstParams p) {
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[rs][c][i] = 0.f;
-    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + 8 * E_ISTR);
+    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + G::HALF);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       bf16x8 n0 = a0, n1 = a1;
       if (kk + 1 < KK) {
         n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
-        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + 8 * E_ISTR);
+        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + G::HALF);
       }
 #pragma unroll
       for (int rs = 0; rs < RS; ++rs) {
@@ -420,24 +271,16 @@ __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
 
 template <int D>
 int launch_est(EstParams& p, int B, hipStream_t stream) {
-  constexpr int NW = 4;
   const int rows_needed = p.out_rows << p.keep_m_log2;
-  dim3 grid((unsigned)((rows_needed + NW * 32 - 1) / (NW * 32)), (unsigned)(B * p.Hq));
+  dim3 grid((unsigned)((rows_needed + 255) / 256), (unsigned)(B * p.Hq));
+  // 256-row workgroups: cut the key range until about 3 workgroups per CU exist (the kernel's occupancy),
+  // keeping at least 8 key tiles per share
   p.ksplit = 1;
-  if (D == 128) {
-    // 256-row workgroups: cut the key range until about 3 workgroups per CU exist (the kernel's occupancy),
-    // keeping at least 8 key tiles per share
-    const int64_t wgs = (int64_t)((rows_needed + 255) / 256) * B * p.Hq;
-    const int tiles = p.Ns_pad / TK;
-    while (p.ksplit < EST_MAX_KSPLIT && wgs * p.ksplit < 3 * 256 && tiles / (p.ksplit * 2) >= 8) p.ksplit *= 2;
-  }
-  if (D == 128) {
-    grid.x = (unsigned)((rows_needed + 255) / 256);
-    grid.z = (unsigned)p.ksplit;
-    hipLaunchKernelGGL(psa_est_gemm128_kernel, grid, dim3(256), 0, stream, p);
-  } else {
-    hipLaunchKernelGGL((psa_est_gemm_kernel<D, NW>), grid, dim3(NW * 64), 0, stream, p);
-  }
+  const int64_t wgs = (int64_t)grid.x * B * p.Hq;
+  const int tiles = p.Ns_pad / TK;
+  while (p.ksplit < EST_MAX_KSPLIT && wgs * p.ksplit < 3 * 256 && tiles / (p.ksplit * 2) >= 8) p.ksplit *= 2;
+  grid.z = (unsigned)p.ksplit;
+  hipLaunchKernelGGL(psa_est_gemm_lds_kernel<D>, grid, dim3(256), 0, stream, p);
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
   hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
