@@ -8,9 +8,9 @@
 //
 // Four kernels:
 //   psa_bwd_delta_kernel   HBM-bound: delta and lse in log2 units (rows without keys get +inf so p = 0)
-//   psa_bwd_dq_kernel      MFMA-bound row walk: the forward's tile schedule; per tile S^T = K Q^T,
+//   psa_bwd_dq_lds_kernel  MFMA-bound row walk: the forward's tile schedule; per tile S^T = K Q^T,
 //                          dP^T = V dO^T, dQ^T += K^T dS^T on bf16 MFMA, operands pooled K/V read directly
-//   psa_bwd_dkdv_kernel    MFMA-bound column walk: one workgroup per (kv head, kv-block, level slot) keeps its
+//   psa_bwd_dkdv_lds_kernel MFMA-bound column walk: one workgroup per (kv head, kv-block, level slot) keeps its
 //                          <= 64 pooled keys in registers and streams the q-blocks that retain this block at
 //                          this level; dK_l, dV_l go to an fp32 workspace (every row written exactly once)
 //   psa_bwd_unpool_kernel  HBM-bound: sums the levels, spreads pooled gradients, folds the pad tail, -> bf16
@@ -70,233 +70,15 @@ __global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------------
-// dQ: row walk
-// ------------------------------------------------------------------------------------------------------
-template <int D>
-struct DqSmem {
-  static constexpr int KST = D * 2 + 16;  // bytes per [key][d] row
-  static constexpr int TST = TK * 2 + 8;  // bytes per [d][key] row
-  static constexpr int ROW_BYTES = TK * KST;
-  static constexpr int T_BYTES = D * TST;
-  static constexpr int TILE_BYTES = 2 * ROW_BYTES + T_BYTES;  // K rows, V rows, K^T
-  static constexpr int OST = D * 2 + 16;
-};
-
-template <int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_kernel(BwdParams p) {
-  constexpr int NT = NW * 64;
-  constexpr int BM = NW * 32;
-  constexpr int CH = D / 8;
-  constexpr int UNITS = 16 * CH;
-  constexpr int PER = (UNITS + NT - 1) / NT;
-  constexpr int KK = D / 16;
-  constexpr int DB = D / 32;
-  using SM = DqSmem<D>;
-  static_assert(BM * SM::OST <= SM::TILE_BYTES, "dQ staging must fit the tile buffers");
-
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* Ks = smem;
-  unsigned char* Vs = smem + SM::ROW_BYTES;
-  unsigned char* Kt = smem + 2 * SM::ROW_BYTES;
-  u32x2* tdesc = (u32x2*)(smem + SM::TILE_BYTES);
-  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
-  __shared__ int s_cnt[4], s_ioff[4], s_toff[5], s_wcnt[4 * (NT / 64)];
-
-  const int I = blockIdx.x % p.Mq;
-  const int bh = blockIdx.x / p.Mq;
-  const int h = bh % p.Hq, b = bh / p.Hq;
-  const int hk = h / (p.Hq / p.Hkv);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, hh = lane >> 5;
-  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal;
-  const float scale_log2 = p.scale_log2;
-
-  int jmax = p.Nk;
-  if (causal) {
-    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << bn_log2) - 1) >> bn_log2);
-    jmax = ce < jmax ? ce : jmax;
-  }
-  const int T = build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, bn_log2, L, causal != 0,
-                                       (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
-
-  // Q and dO fragments of this wave's 32 rows (B operands), per-row delta and lse
-  const int q_idx = I * BM + wave * 32 + l32;
-  const int qr = q_idx < L ? q_idx : L - 1;
-  bf16x8 qf[KK], dof[KK];
-  {
-    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
-    const bf16_t* dp_ = p.dout + b * p.do_sb + h * p.do_sh + (int64_t)qr * p.do_sl + hh * 8;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      qf[kk] = *(const bf16x8*)(qp + kk * 16);
-      dof[kk] = *(const bf16x8*)(dp_ + kk * 16);
-    }
-  }
-  const float delta = q_idx < L ? p.delta[(int64_t)bh * L + q_idx] : 0.f;
-  const float lse2 = q_idx < L ? p.lse2[(int64_t)bh * L + q_idx] : INFINITY;
-
-  const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
-  const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
-  const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
-  const int64_t npad = p.npad;
-  const uint32_t k_strb = (uint32_t)p.k_sl * 2u, v_strb = (uint32_t)p.v_sl * 2u;
-  const bf16_t *kpool = p.kp, *vpool = p.vp;
-
-  u32x4 kreg[PER][4], vreg[PER][4];
-  auto load_tile = [&](int t) __attribute__((always_inline)) {
-    const TileRef r = tile_ref(tdesc, ids, t, bn_log2);
-    const int64_t prow = pool_row_offset(r.lv, BHkv, bhk, npad) * D;
-    const char* kbase = r.lv == 0 ? kb0 : (const char*)(kpool + prow);
-    const char* vbase = r.lv == 0 ? vb0 : (const char*)(vpool + prow);
-    const uint32_t ks = r.lv == 0 ? k_strb : (uint32_t)(D * 2);
-    const uint32_t vs = r.lv == 0 ? v_strb : (uint32_t)(D * 2);
-    const int lim = r.lv == 0 ? L : 0x7fffffff;
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u & 15) * 4, ch = u >> 4;  // neighbouring lanes walk along the key quads of one chunk
-      const int src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, L);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int src = src0 + i;
-        src = (src0 >= 0 && src < lim) ? src : 0;  // empty slots: finite data, masked below
-        kreg[u_][i] = *(const u32x4*)(kbase + ((uint32_t)src * ks + (uint32_t)(ch * 16)));
-        vreg[u_][i] = *(const u32x4*)(vbase + ((uint32_t)src * vs + (uint32_t)(ch * 16)));
-      }
-    }
-  };
-  auto store_tile = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int u_ = 0; u_ < PER; ++u_) {
-      const int u = tid + u_ * NT;
-      if (UNITS % NT != 0 && u >= UNITS) break;
-      const int r0 = (u & 15) * 4, ch = u >> 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *(u32x4*)(Ks + (r0 + i) * SM::KST + ch * 16) = kreg[u_][i];
-        *(u32x4*)(Vs + (r0 + i) * SM::KST + ch * 16) = vreg[u_][i];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {  // K^T: 4 keys x 8 channels -> 8 channels x 4 keys
-        u32x2 e0, e1;
-        e0[0] = __builtin_amdgcn_perm(kreg[u_][1][j], kreg[u_][0][j], 0x05040100u);
-        e0[1] = __builtin_amdgcn_perm(kreg[u_][3][j], kreg[u_][2][j], 0x05040100u);
-        e1[0] = __builtin_amdgcn_perm(kreg[u_][1][j], kreg[u_][0][j], 0x07060302u);
-        e1[1] = __builtin_amdgcn_perm(kreg[u_][3][j], kreg[u_][2][j], 0x07060302u);
-        *(u32x2*)(Kt + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
-        *(u32x2*)(Kt + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
-      }
-    }
-  };
-
-  f32x16 acc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-
-  if (T > 0) load_tile(0);
-  for (int t = 0; t < T; ++t) {
-    __syncthreads();
-    store_tile();
-    __syncthreads();
-    const TileRef r = tile_ref(tdesc, ids, t, bn_log2);
-    if (t + 1 < T) load_tile(t + 1);
-
-    f32x16 s[2], dp[2];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[c][i] = 0.f;
-        dp[c][i] = 0.f;
-      }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const bf16x8 ka = *(const bf16x8*)(Ks + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
-        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s[c], 0, 0, 0);
-        const bf16x8 va = *(const bf16x8*)(Vs + (c * 32 + l32) * SM::KST + hh * 16 + kk * 32);
-        dp[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp[c], 0, 0, 0);
-      }
-    }
-    if (r.masked) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int r0 = c * 32 + g * 8 + hh * 4;
-          int src0 = -1;
-          if (r0 < r.nvalid) src0 = slot_src(r.lv, r.lt, r0, r.sbs_log2, r.cnt, r.ids, L);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const bool in_tile = src0 >= 0 && (r0 + e) < r.nvalid;
-            const bool visible = !causal || ((((int64_t)(src0 + e) + 1) << r.lv) - 1 <= (int64_t)q_idx);
-            const float sv = s[c][g * 4 + e];
-            s[c][g * 4 + e] = (in_tile && visible) ? sv : -INFINITY;
-          }
-        }
-    }
-    const float nb = (float)r.lv - lse2;
-    uint32_t pk[2][8];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        const float p0 = fast_exp2(__builtin_fmaf(s[c][i], scale_log2, nb));
-        const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], scale_log2, nb));
-        pk[c][i >> 1] = pack_bf16x2(p0 * (dp[c][i] - delta), p1 * (dp[c][i + 1] - delta));
-      }
-    // dQ^T += K^T dS^T
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
-        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
-        const int key0 = c * 32 + g * 16 + hh * 4;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const unsigned char* kr = Kt + (db * 32 + l32) * SM::TST + key0 * 2;
-          const u32x2 lo = *(const u32x2*)(kr);
-          const u32x2 hi = *(const u32x2*)(kr + 16);
-          u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
-        }
-      }
-  }
-
-  __syncthreads();
-  unsigned char* Os = smem;
-  const float scale = p.scale;
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      u32x2 w;
-      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * scale, acc[db][g * 4 + 1] * scale);
-      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * scale, acc[db][g * 4 + 3] * scale);
-      *(u32x2*)(Os + (wave * 32 + l32) * SM::OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
-    }
-  __syncthreads();
-  bf16_t* ob = p.dq + b * p.dq_sb + h * p.dq_sh;
-  for (int u = tid; u < BM * CH; u += NT) {
-    const int rr = u / CH, ch = u % CH;
-    const int row = I * BM + rr;
-    if (row < L) *(u32x4*)(ob + (int64_t)row * p.dq_sl + ch * 8) = *(const u32x4*)(Os + rr * SM::OST + ch * 16);
-  }
-}
-
-// ------------------------------------------------------------------------------------------------------
 // dQ row walk, head dim 128: the forward's data path.  K and V tiles are copied from global memory straight
 // into double-buffered LDS tiles (layout: psa_tiles.h), one barrier per tile; S^T = K Q^T and dP^T = V dO^T
 // read them row-wise (128-bit reads), dQ^T += K^T dS^T reads the K tile through the transposing LDS load.
 // ------------------------------------------------------------------------------------------------------
-template <int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) {
-  constexpr int D = 128, NT = NW * 64, BM = NW * 32, CH = D / 8, KK = D / 16, DB = D / 32;
+template <int D, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p) {
+  using G = LtGeom<D>;
+  constexpr int LT_TILE = G::TILE;
+  constexpr int NT = NW * 64, BM = NW * 32, CH = D / 8, KK = D / 16, DB = D / 32;
   constexpr int G16 = 4 / NW;
   constexpr int OST = D * 2 + 16;
   static_assert(BM * OST <= 4 * LT_TILE, "dQ staging must fit the tile buffers");
@@ -347,16 +129,16 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) 
   kvs.k_strb = (uint32_t)p.k_sl * 2u; kvs.v_strb = (uint32_t)p.v_sl * 2u;
   kvs.BHkv = (int64_t)p.B * p.Hkv; kvs.bhk = (int64_t)b * p.Hkv + hk; kvs.npad = p.npad;
   kvs.bn_log2 = bn_log2; kvs.L = L;
-  const uint32_t f_chunk = lt_fetch_chunk<128>(lane);
+  const uint32_t f_chunk = lt_fetch_chunk<D>(lane);
   uint32_t r_off[2], t_off[2];
-  lt_row_operand<128>(l32, hh, r_off);  // tile rows l32 (+32): r_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
-  lt_tr_operand<128>(lane, t_off);      // K^T: t_off[s] + 64 * db + 4 * LT_ISTR * (16-key group)
+  lt_row_operand<D>(l32, hh, r_off);  // tile rows l32 (+32): r_off[kk & 1] + 64 * (kk >> 1) (+ 8 blocks)
+  lt_tr_operand<D>(lane, t_off);      // K^T: t_off[s] + 64 * db + 4 * LT_ISTR * (16-key group)
 
   auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
     TileSrc<G16> ts;
-    lt_tile_src<128, G16>(kvs, tdesc, ids, t, wave, lane, ts);
-    lt_issue_rows<128, G16>(smem + stage * LT_TILE, ts.kbase, ts.kstr, ts.lim, ts.src0, wave, f_chunk);
-    lt_issue_rows<128, G16>(smem + (2 + stage) * LT_TILE, ts.vbase, ts.vstr, ts.lim, ts.src0, wave, f_chunk);
+    lt_tile_src<D, G16>(kvs, tdesc, ids, t, wave, lane, ts);
+    lt_issue_rows<D, G16>(smem + stage * LT_TILE, ts.kbase, ts.kstr, ts.lim, ts.src0, wave, f_chunk);
+    lt_issue_rows<D, G16>(smem + (2 + stage) * LT_TILE, ts.vbase, ts.vstr, ts.lim, ts.src0, wave, f_chunk);
   };
 
   f32x16 acc[DB];
@@ -383,9 +165,9 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) 
     for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        const bf16x8 ka = *(PSA_LDS(const bf16x8))(Ks + r_off[kk & 1] + (kk >> 1) * 64 + c * 8 * LT_ISTR);
+        const bf16x8 ka = *(PSA_LDS(const bf16x8))(Ks + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
         s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s[c], 0, 0, 0);
-        const bf16x8 va = *(PSA_LDS(const bf16x8))(Vs + r_off[kk & 1] + (kk >> 1) * 64 + c * 8 * LT_ISTR);
+        const bf16x8 va = *(PSA_LDS(const bf16x8))(Vs + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
         dp[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp[c], 0, 0, 0);
       }
     }
@@ -432,8 +214,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) 
       const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[0] + db * 64 + cg * (4 * LT_ISTR))));
-        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[1] + db * 64 + cg * (4 * LT_ISTR))));
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[0] + db * 64 + cg * G::GROUP)));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[1] + db * 64 + cg * G::GROUP)));
         u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
         acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
       }
@@ -485,18 +267,6 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq128_kernel(BwdParams p) 
   }
 }
 
-// ------------------------------------------------------------------------------------------------------
-// dK, dV: column walk
-// ------------------------------------------------------------------------------------------------------
-template <int D>
-struct KvSmem {
-  static constexpr int RST = D * 2 + 16;   // bytes per [q][d] row
-  static constexpr int TST = 64 * 2 + 8;   // bytes per [d][q] row (64 query rows per step)
-  static constexpr int ROW_BYTES = 64 * RST;
-  static constexpr int T_BYTES = D * TST;
-  static constexpr int STAGE_BYTES = 2 * ROW_BYTES + 2 * T_BYTES;  // Q rows, dO rows, Q^T, dO^T
-};
-
 // slot -> (level, 64-key part inside the block); slots of a block: max(1, (bn>>lv)/64) per level
 __device__ __forceinline__ void decode_slot(int slot, int bn_log2, int& lv, int& part) {
   lv = 0;
@@ -507,257 +277,6 @@ __device__ __forceinline__ void decode_slot(int slot, int bn_log2, int& lv, int&
     ++lv;
   }
   part = slot;
-}
-
-template <int D>
-__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_kernel(BwdParams p, int slots_per_block) {
-  constexpr int NT = 256;
-  constexpr int CH = D / 8;
-  constexpr int UNITS = 16 * CH;
-  constexpr int PER = (UNITS + NT - 1) / NT;
-  constexpr int KK = D / 16;
-  constexpr int DB = D / 32;
-  using SM = KvSmem<D>;
-
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* Qs = smem;
-  unsigned char* Os = smem + SM::ROW_BYTES;
-  unsigned char* Qt = smem + 2 * SM::ROW_BYTES;
-  unsigned char* Ot = smem + 2 * SM::ROW_BYTES + SM::T_BYTES;
-  float* s_lse = (float*)(smem + SM::STAGE_BYTES);  // [64]
-  float* s_del = s_lse + 64;                        // [64]
-  uint32_t* qlist = (uint32_t*)(s_del + 64);        // [n_rep * Mq]  (head in group << 16 | q-block)
-  __shared__ int s_nq;
-
-  const int slot = blockIdx.x % slots_per_block;
-  const int J = blockIdx.x / slots_per_block;
-  const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
-  const int n_rep = p.Hq / p.Hkv;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, hh = lane >> 5;
-  const int kh = wave & 1, qh = wave >> 1;
-  const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal, bm = p.bm, Mq = p.Mq;
-
-  int lv, part;
-  decode_slot(slot, bn_log2, lv, part);
-  const int sbs = 1 << (bn_log2 - lv);            // pooled keys of this block at this level
-  const int nkeys = sbs < 64 ? sbs : 64;
-  const int64_t key_row0 = ((int64_t)J << (bn_log2 - lv)) + part * 64;  // first pooled row of this workgroup
-  const int64_t n_lv = p.npad >> lv;
-  int key_valid = nkeys;                          // level 0: rows past L do not exist
-  if (lv == 0) {
-    const int64_t rem = (int64_t)L - key_row0;
-    key_valid = rem < nkeys ? (rem > 0 ? (int)rem : 0) : nkeys;
-  }
-
-  // ---- list of (head in group, q-block) that retain block J at this level -------------------------
-  if (wave == 0) {
-    int n = 0;
-    const int total = n_rep * Mq;
-    for (int e0 = 0; e0 < total; e0 += 64) {
-      const int e = e0 + lane;
-      bool on = false;
-      if (e < total) {
-        const int hl = e / Mq, I = e % Mq;
-        const int h = hk * n_rep + hl;
-        int level = p.map ? load_map(p.map, (((int64_t)b * p.Hq + h) * Mq + I) * p.Nk + J, p.map_elem) : 1;
-        if (causal) {
-          const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
-          if (J >= ce) level = 0;
-        }
-        on = level == (1 << lv);
-      }
-      const uint64_t bal = __ballot(on);
-      if (on) qlist[n + __popcll(bal & ((1ull << lane) - 1ull))] = ((uint32_t)(e / Mq) << 16) | (uint32_t)(e % Mq);
-      n += __popcll(bal);
-    }
-    if (lane == 0) s_nq = n;
-  }
-  __syncthreads();
-  const int nq = s_nq;
-
-  // ---- this wave's 32 keys: K and V fragments (B operands) --------------------------------------------
-  const int key_local = kh * 32 + l32;
-  bf16x8 kf[KK], vf[KK];
-  {
-    int64_t row = key_row0 + (key_local < key_valid ? key_local : 0);
-    if (key_valid == 0) row = 0;
-    const bf16_t *kp_, *vp_;
-    if (lv == 0 || p.kp == nullptr) {
-      // without a level map there are no pooled buffers: the workgroups of the pooled levels have an empty
-      // q-block list and only write zeros, whatever they load here
-      kp_ = p.k + b * p.k_sb + hk * p.k_sh + (lv == 0 ? row : 0) * p.k_sl;
-      vp_ = p.v + b * p.v_sb + hk * p.v_sh + (lv == 0 ? row : 0) * p.v_sl;
-    } else {
-      const int64_t off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + row) * D;
-      kp_ = p.kp + off;
-      vp_ = p.vp + off;
-    }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      kf[kk] = *(const bf16x8*)(kp_ + kk * 16 + hh * 8);
-      vf[kk] = *(const bf16x8*)(vp_ + kk * 16 + hh * 8);
-    }
-  }
-  const bool key_ok = key_local < key_valid;
-  const int64_t key_up = ((key_row0 + key_local + 1) << lv) - 1;  // last token the pooled key covers
-
-  f32x16 dk[DB], dv[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      dk[db][i] = 0.f;
-      dv[db][i] = 0.f;
-    }
-  const float scale_log2 = p.scale_log2;
-  const float bias = (float)lv;
-  const int steps_per_block = bm / 64;
-
-  if (key_valid > 0) {
-    for (int e = 0; e < nq; ++e) {
-      const uint32_t ent = qlist[e];
-      const int h = hk * n_rep + (int)(ent >> 16), I = (int)(ent & 0xffff);
-      const int64_t bh = (int64_t)b * p.Hq + h;
-      const bool diag = causal && ((((int64_t)J + 1) << bn_log2) - 1 > (int64_t)I * bm);
-      for (int st = 0; st < steps_per_block; ++st) {
-        const int q0 = I * bm + st * 64;
-        if (q0 >= L) break;
-        __syncthreads();  // previous step's reads of the staging buffers are done
-        // stage 64 rows of Q and dO in both layouts
-#pragma unroll
-        for (int u_ = 0; u_ < PER; ++u_) {
-          const int u = tid + u_ * NT;
-          if (UNITS % NT != 0 && u >= UNITS) break;
-          const int r0 = (u & 15) * 4, ch = u >> 4;
-          u32x4 qreg[4], oreg[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            int row = q0 + r0 + i;
-            row = row < L ? row : L - 1;  // rows past L: p is forced to 0 through lse = +inf
-            qreg[i] = *(const u32x4*)(p.q + b * p.q_sb + h * p.q_sh + (int64_t)row * p.q_sl + ch * 8);
-            oreg[i] = *(const u32x4*)(p.dout + b * p.do_sb + h * p.do_sh + (int64_t)row * p.do_sl + ch * 8);
-            *(u32x4*)(Qs + (r0 + i) * SM::RST + ch * 16) = qreg[i];
-            *(u32x4*)(Os + (r0 + i) * SM::RST + ch * 16) = oreg[i];
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            u32x2 e0, e1;
-            e0[0] = __builtin_amdgcn_perm(qreg[1][j], qreg[0][j], 0x05040100u);
-            e0[1] = __builtin_amdgcn_perm(qreg[3][j], qreg[2][j], 0x05040100u);
-            e1[0] = __builtin_amdgcn_perm(qreg[1][j], qreg[0][j], 0x07060302u);
-            e1[1] = __builtin_amdgcn_perm(qreg[3][j], qreg[2][j], 0x07060302u);
-            *(u32x2*)(Qt + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
-            *(u32x2*)(Qt + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
-            e0[0] = __builtin_amdgcn_perm(oreg[1][j], oreg[0][j], 0x05040100u);
-            e0[1] = __builtin_amdgcn_perm(oreg[3][j], oreg[2][j], 0x05040100u);
-            e1[0] = __builtin_amdgcn_perm(oreg[1][j], oreg[0][j], 0x07060302u);
-            e1[1] = __builtin_amdgcn_perm(oreg[3][j], oreg[2][j], 0x07060302u);
-            *(u32x2*)(Ot + (ch * 8 + 2 * j) * SM::TST + r0 * 2) = e0;
-            *(u32x2*)(Ot + (ch * 8 + 2 * j + 1) * SM::TST + r0 * 2) = e1;
-          }
-        }
-        if (tid < 64) {
-          const int row = q0 + tid;
-          s_lse[tid] = row < L ? p.lse2[bh * L + row] : INFINITY;
-          s_del[tid] = row < L ? p.delta[bh * L + row] : 0.f;
-        }
-        __syncthreads();
-
-        // S = Q K^T and dP = dO V^T for this wave's (32 q) x (32 keys): lane = key column, registers = q rows
-        f32x16 s, dp;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          s[i] = 0.f;
-          dp[i] = 0.f;
-        }
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          const bf16x8 qa = *(const bf16x8*)(Qs + (qh * 32 + l32) * SM::RST + hh * 16 + kk * 32);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
-          const bf16x8 oa = *(const bf16x8*)(Os + (qh * 32 + l32) * SM::RST + hh * 16 + kk * 32);
-          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[kk], dp, 0, 0, 0);
-        }
-        uint32_t pk[8], dsk[8];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int qq = qh * 32 + g * 8 + hh * 4;
-          const f32x4 l4 = *(const f32x4*)(s_lse + qq);
-          const f32x4 d4 = *(const f32x4*)(s_del + qq);
-          float pv[4], dsv[4];
-#pragma unroll
-          for (int e2 = 0; e2 < 4; ++e2) {
-            float pe = fast_exp2(__builtin_fmaf(s[g * 4 + e2], scale_log2, bias - l4[e2]));
-            bool ok = key_ok;
-            if (diag) ok = ok && (key_up <= (int64_t)(q0 + qq + e2));
-            pe = ok ? pe : 0.f;
-            pv[e2] = pe;
-            dsv[e2] = pe * (dp[g * 4 + e2] - d4[e2]);
-          }
-          pk[g * 2] = pack_bf16x2(pv[0], pv[1]);
-          pk[g * 2 + 1] = pack_bf16x2(pv[2], pv[3]);
-          dsk[g * 2] = pack_bf16x2(dsv[0], dsv[1]);
-          dsk[g * 2 + 1] = pack_bf16x2(dsv[2], dsv[3]);
-        }
-        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over this wave's 32 query rows, 16 at a time)
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
-          u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
-          const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
-          const int qq0 = qh * 32 + g * 16 + hh * 4;
-#pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            const unsigned char* orow = Ot + (db * 32 + l32) * SM::TST + qq0 * 2;
-            const u32x2 olo = *(const u32x2*)(orow), ohi = *(const u32x2*)(orow + 16);
-            u32x4 oa = {olo[0], olo[1], ohi[0], ohi[1]};
-            dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, oa), pfrag, dv[db], 0, 0, 0);
-            const unsigned char* qrow = Qt + (db * 32 + l32) * SM::TST + qq0 * 2;
-            const u32x2 qlo = *(const u32x2*)(qrow), qhi = *(const u32x2*)(qrow + 16);
-            u32x4 qa2 = {qlo[0], qlo[1], qhi[0], qhi[1]};
-            dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qa2), sfrag, dk[db], 0, 0, 0);
-          }
-        }
-      }
-    }
-  }
-
-  // ---- combine the two query halves and write this workgroup's rows of the level buffers ------------
-  __syncthreads();
-  float* red = (float*)smem;  // [2 key halves][2 tensors][DB*16][64 lanes]
-  if (qh == 1) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane] = dk[db][i];
-        red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane] = dv[db][i];
-      }
-  }
-  __syncthreads();
-  if (qh == 0 && key_local < nkeys) {
-    const int64_t lvl_off = (pool_row_offset(lv, (int64_t)p.B * p.Hkv, bhk, p.npad) + (lv == 0 ? (int64_t)p.B * p.Hkv * 0 : 0));
-    // level buffers: level 0 first ([BHkv, npad, D]), then levels 1..3 like the pooled K/V buffers
-    const int64_t base_rows = lv == 0 ? bhk * p.npad : (int64_t)p.B * p.Hkv * p.npad + lvl_off;
-    float* wk = p.wk + (base_rows + key_row0 + key_local) * D;
-    float* wv = p.wv + (base_rows + key_row0 + key_local) * D;
-    const float scale = p.scale;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 a, c2;
-#pragma unroll
-        for (int e2 = 0; e2 < 4; ++e2) {
-          const int i = g * 4 + e2;
-          a[e2] = (dk[db][i] + red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane]) * scale;
-          c2[e2] = dv[db][i] + red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane];
-        }
-        *(f32x4*)(wk + db * 32 + g * 8 + hh * 4) = a;
-        *(f32x4*)(wv + db * 32 + g * 8 + hh * 4) = c2;
-      }
-  }
-  (void)n_lv;
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -838,11 +357,13 @@ __global__ __launch_bounds__(256) void psa_bwd_colsort_kernel(const int32_t* cos
 // kernel; the row operands (S = Q K^T, dP = dO V^T) are 128-bit LDS reads and the transposed operands
 // (dV^T += dO^T P, dK^T += Q^T dS) come from the same tiles through the transposing LDS load.
 // ------------------------------------------------------------------------------------------------------
-constexpr int B_ISTR = LT_ISTR;  // bytes between the 4-row blocks of a tile
-constexpr int B_TILE = LT_TILE;  // 64 rows x 256 bytes, padded
+constexpr int B_ISTR = LT_ISTR;  // bytes between the blocks of a tile
 
-__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, int slots_per_block, const int32_t* order) {
-  constexpr int D = 128, KK = D / 16, DB = D / 32;
+template <int D>
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slots_per_block, const int32_t* order) {
+  using G = LtGeom<D>;
+  constexpr int KK = D / 16, DB = D / 32, RPL = G::RPL;
+  constexpr int B_TILE = G::TILE;
   extern __shared__ __align__(16) unsigned char smem[];
   // stage s: Q tile at 2*s*B_TILE, dO tile at (2*s + 1)*B_TILE
   float* s_lse = (float*)(smem + 4 * B_TILE);  // [2 stages][64]
@@ -931,11 +452,11 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
   // ---- lane-invariant LDS addressing (tile layout: see the forward kernel) ---------------------------
   // copy: wave w fills the 16-row group w of both tiles; lane (fq = lane/16, pos = lane%16) of block n writes
   // row fq of that block, i.e. tile row 16w + 4fq + n, chunk pos ^ fq
-  const uint32_t f_chunk = lt_fetch_chunk<128>(lane);
-  const int f_row = wave * 16 + lt_fetch_row<128>(lane);
+  const uint32_t f_chunk = lt_fetch_chunk<D>(lane);
+  const int f_row = wave * 16 + lt_fetch_row<D>(lane);
   uint32_t r_off[2], t_off[2];
-  lt_row_operand<128>(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
-  lt_tr_operand<128>(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
+  lt_row_operand<D>(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
+  lt_tr_operand<D>(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -978,22 +499,22 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
     if (q0 + 64 <= L) {
       const uint32_t qo = (uint32_t)r0 * q_strb + f_chunk, oo = (uint32_t)r0 * do_strb + f_chunk;
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
+      for (int n = 0; n < RPL; ++n) {
         __builtin_amdgcn_global_load_lds(qb + (uint64_t)(n * q_strb) + qo,
-                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(ob + (uint64_t)(n * do_strb) + oo,
-                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
       }
     } else {
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
+      for (int n = 0; n < RPL; ++n) {
         int row = r0 + n;
         row = row < L ? row : L - 1;
         row = row > 0 ? row : 0;
         __builtin_amdgcn_global_load_lds(qb + ((uint32_t)row * q_strb + f_chunk),
-                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(ob + ((uint32_t)row * do_strb + f_chunk),
-                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * 4 + n) * B_ISTR), 16, 0, 0);
+                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
       }
     }
   };
@@ -1056,7 +577,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv128_kernel(BwdParams p, in
       u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
       u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
       const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
-      const int grp = (2 * qh + g) * (4 * B_ISTR);
+      const int grp = (2 * qh + g) * G::GROUP;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const u32x2 olo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[0] + db * 64 + grp)));
@@ -1270,10 +791,10 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       return PSA_OK;
     };
     int rc;
-    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq128_kernel<4>, (size_t)4 * LT_TILE, 4);
-    else if (D == 128) rc = launch(psa_bwd_dq128_kernel<2>, (size_t)4 * LT_TILE, 2);
-    else if (block_m == 128) rc = launch(psa_bwd_dq_kernel<64, 4>, DqSmem<64>::TILE_BYTES, 4);
-    else rc = launch(psa_bwd_dq_kernel<64, 2>, DqSmem<64>::TILE_BYTES, 2);
+    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 4>, (size_t)4 * LtGeom<128>::TILE, 4);
+    else if (D == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 2>, (size_t)4 * LtGeom<128>::TILE, 2);
+    else if (block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<64, 4>, (size_t)4 * LtGeom<64>::TILE, 4);
+    else rc = launch(psa_bwd_dq_lds_kernel<64, 2>, (size_t)4 * LtGeom<64>::TILE, 2);
     PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: sequence too long for the on-chip schedule (LDS)");
     rc = psa_check_launch("psa_bwd (dQ)");
     if (rc != PSA_OK) return rc;
@@ -1284,31 +805,27 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     const int n_rep = Hq / Hkv;
     const int64_t n_wg = (int64_t)B * Hkv * Nk * spb;
     PSA_REQUIRE(n_wg < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
-    size_t shmem = (D == 128 ? (size_t)4 * LT_TILE + 256 * sizeof(float) : KvSmem<64>::STAGE_BYTES + 128 * sizeof(float)) +
-                   (size_t)n_rep * Mq * 4;
+    size_t shmem = (size_t)4 * (D == 128 ? LtGeom<128>::TILE : LtGeom<64>::TILE) + 256 * sizeof(float) + (size_t)n_rep * Mq * 4;
     const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
     if (shmem < red) shmem = red;
     PSA_REQUIRE(shmem <= 160 * 1024, PSA_ERR_UNSUPPORTED, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
-    if (D == 128) {
-      // longest columns first (needs a level map; the order lives behind lse2 in the workspace)
-      int32_t* order = nullptr;
-      if (map != nullptr && n_wg > 32) {
-        int32_t* cost = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
-        order = cost + n_wg;
-        hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, spb, cost);
-        if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
-        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(256), 0, st, cost, (int)n_wg, order);
-        if (int e = psa_check_launch("psa_bwd (column order)")) return e;
-      }
-      PSA_REQUIRE(hipFuncSetAttribute((const void*)psa_bwd_dkdv128_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) == hipSuccess,
-                  PSA_ERR_LAUNCH, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
-      hipLaunchKernelGGL(psa_bwd_dkdv128_kernel, dim3((unsigned)n_wg), dim3(256), shmem, st, p, spb, order);
-    } else {
-      PSA_REQUIRE(shmem <= 48 * 1024 || hipFuncSetAttribute((const void*)psa_bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                            (int)shmem) == hipSuccess,
-                  PSA_ERR_LAUNCH, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
-      hipLaunchKernelGGL(psa_bwd_dkdv_kernel<64>, dim3((unsigned)(Nk * spb), (unsigned)(B * Hkv)), dim3(256), shmem, st, p, spb);
+    // longest columns first (needs a level map; the order lives behind lse2 in the workspace)
+    int32_t* order = nullptr;
+    if (map != nullptr && n_wg > 32) {
+      int32_t* cost = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
+      order = cost + n_wg;
+      hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, spb, cost);
+      if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
+      hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(256), 0, st, cost, (int)n_wg, order);
+      if (int e = psa_check_launch("psa_bwd (column order)")) return e;
     }
+    auto launch = [&](auto kern) -> int {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) return PSA_ERR_LAUNCH;
+      hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3(256), shmem, st, p, spb, order);
+      return PSA_OK;
+    };
+    const int rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128>) : launch(psa_bwd_dkdv_lds_kernel<64>);
+    PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
     const int rc = psa_check_launch("psa_bwd (dK/dV)");
     if (rc != PSA_OK) return rc;
   }
