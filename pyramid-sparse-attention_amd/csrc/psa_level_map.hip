@@ -394,26 +394,42 @@ extern "C" int psa_map_min_cap(void* map, int map_elem_bytes, const int32_t* cap
 // ---------------------------------------------------------------------------------------
 // density = mean(1/level)
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void psa_density_kernel(const void* map, int map_elem, int Mq, int Nk, int causal, int BH,
-                                                          float* out) {
-  __shared__ float s_part[4];
+__global__ __launch_bounds__(1024) void psa_density_kernel(const void* map, int map_elem, int Mq, int Nk, int causal, int BH,
+                                                           float* out) {
+  __shared__ float s_part[16];
   const int64_t bh = blockIdx.x;
   const int64_t n = (int64_t)Mq * Nk;
+  const int tid = threadIdx.x;
   // counts per level are exact integers; 1/level sums are exact in fp32 up to 2^24/8 blocks
   int c1 = 0, c2 = 0, c4 = 0, c8 = 0;
-  for (int r = 0; r < Mq; ++r) {
-    const int cend = causal ? (r + 1 < Nk ? r + 1 : Nk) : Nk;
-    for (int c = threadIdx.x; c < cend; c += 256) {
-      const int lv = load_map(map, bh * n + (int64_t)r * Nk + c, map_elem);
-      c1 += lv == 1; c2 += lv == 2; c4 += lv == 4; c8 += lv == 8;
+  auto count = [&](int lv, int64_t idx) {
+    if (causal) {
+      const int64_t r = idx / Nk, c = idx - r * Nk;
+      if (c > r) return;
+    }
+    c1 += lv == 1; c2 += lv == 2; c4 += lv == 4; c8 += lv == 8;
+  };
+  const unsigned char* base = (const unsigned char*)map + bh * n * map_elem;
+  const int epu = 16 / map_elem;  // map entries per 16-byte load
+  const int64_t units = (((uintptr_t)base & 15) == 0) ? n / epu : 0;
+  for (int64_t u = tid; u < units; u += 1024) {
+    const u32x4 w = *(const u32x4*)(base + u * 16);
+    if (map_elem == 1) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) count((int)(signed char)((w[e >> 2] >> ((e & 3) * 8)) & 0xff), u * 16 + e);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) count((int)w[e], u * 4 + e);
     }
   }
+  for (int64_t idx = units * epu + tid; idx < n; idx += 1024) count(load_map(map, bh * n + idx, map_elem), idx);
   float v = (float)c1 + 0.5f * (float)c2 + 0.25f * (float)c4 + 0.125f * (float)c8;
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
+  if ((tid & 63) == 0) s_part[tid >> 6] = v;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const float tot = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+  if (tid == 0) {
+    float tot = 0.f;
+    for (int w = 0; w < 16; ++w) tot += s_part[w];  // exact: multiples of 1/8 below 2^21
     const double cnt = causal ? ((double)(Mq < Nk ? Mq : Nk) * ((Mq < Nk ? Mq : Nk) + 1) / 2.0 +
                                  (Mq > Nk ? (double)(Mq - Nk) * Nk : 0.0))
                               : (double)n;
@@ -434,7 +450,7 @@ extern "C" int psa_density(const void* map, int map_elem_bytes, int64_t bh, int 
   PSA_REQUIRE(map && density_out, PSA_ERR_ARG, "psa_density: null pointer");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_density: map_elem_bytes must be 1 or 4");
   PSA_REQUIRE(bh > 0 && bh < (1 << 30) && Mq > 0 && Nk > 0, PSA_ERR_ARG, "psa_density: bad sizes");
-  hipLaunchKernelGGL(psa_density_kernel, dim3((unsigned)bh), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes, Mq,
+  hipLaunchKernelGGL(psa_density_kernel, dim3((unsigned)bh), dim3(1024), 0, (hipStream_t)stream, map, map_elem_bytes, Mq,
                      Nk, causal, (int)bh, density_out);
   hipLaunchKernelGGL(psa_density_mean_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, density_out, (int)bh);
   return psa_check_launch("psa_density");
