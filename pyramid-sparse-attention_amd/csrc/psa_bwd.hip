@@ -500,10 +500,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
       const uint32_t qo = (uint32_t)r0 * q_strb + f_chunk, oo = (uint32_t)r0 * do_strb + f_chunk;
 #pragma unroll
       for (int n = 0; n < RPL; ++n) {
-        __builtin_amdgcn_global_load_lds(qb + (uint64_t)(n * q_strb) + qo,
-                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(ob + (uint64_t)(n * do_strb) + oo,
-                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
+        psa_tiles::lds_copy16(qb + (uint64_t)(n * q_strb), qo, psa_tiles::lds_addr_of(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR));
+        psa_tiles::lds_copy16(ob + (uint64_t)(n * do_strb), oo, psa_tiles::lds_addr_of(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR));
       }
     } else {
 #pragma unroll
@@ -511,10 +509,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
         int row = r0 + n;
         row = row < L ? row : L - 1;
         row = row > 0 ? row : 0;
-        __builtin_amdgcn_global_load_lds(qb + ((uint32_t)row * q_strb + f_chunk),
-                                         (PSA_LDS(void))(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(ob + ((uint32_t)row * do_strb + f_chunk),
-                                         (PSA_LDS(void))(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR), 16, 0, 0);
+        psa_tiles::lds_copy16(qb, (uint32_t)row * q_strb + f_chunk, psa_tiles::lds_addr_of(smem + 2 * stage * B_TILE + (wave * RPL + n) * B_ISTR));
+        psa_tiles::lds_copy16(ob, (uint32_t)row * do_strb + f_chunk, psa_tiles::lds_addr_of(smem + (2 * stage + 1) * B_TILE + (wave * RPL + n) * B_ISTR));
       }
     }
   };

@@ -111,8 +111,7 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
         }
         src = src < Lk ? src : Lk - 1;
       }
-      __builtin_amdgcn_global_load_lds(kb + ((uint32_t)src * kstrb + f_chunk),
-                                       (PSA_LDS(void))(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR), 16, 0, 0);
+      psa_tiles::lds_copy16(kb, (uint32_t)src * kstrb + f_chunk, psa_tiles::lds_addr_of(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR));
     }
   };
   // K operand of k-step kk for tile slots l32 and l32 + 32: k_off[kk & 1] + 64 * (kk >> 1) (+ G::HALF)

@@ -1,7 +1,8 @@
 // Pyramid sparse attention forward (non-causal and causal) on bf16 MFMA.
 //
-// One workgroup per (batch, head, q-block of BM = 32*NW rows); every wave owns 32 query rows; two workgroups
-// per CU.
+// psa_fwd_lds_kernel: one workgroup per (batch, head, q-block of BM = 32*NW rows); every wave owns 32 query rows;
+// two workgroups per CU.  psa_fwd_pp_kernel (head dim 128, 128-row q-blocks, the usual case): two rows per
+// workgroup of 8 waves, see there.  Both share the points below.
 //
 //  * The workgroup first compacts its row of the level map into four per-level lists of kv-block ids in LDS
 //    (ballot + popcount, ascending block order - deterministic) and a list of tile descriptors.
@@ -33,6 +34,9 @@
 
 namespace {
 
+#ifndef PSA_FWD_ONE_GROUP
+#define PSA_FWD_ONE_GROUP 0
+#endif
 constexpr int TK = 64;              // pooled keys per tile
 constexpr float LAZY_THRESHOLD = 8.f;  // log2 units the running max may lag behind
 
@@ -50,6 +54,7 @@ struct FwdParams {
   int causal;
   int total_wg, wg_chunk, wg_groups;  // rows are dealt in wg_groups groups of wg_chunk; group g runs on XCD g % 8
   int max_tiles;
+  int grp_bytes;  // two-group kernel: LDS bytes of one group (tile buffers + schedule)
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
 };
 
@@ -334,6 +339,427 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   }
 }
 
+// ---- two-group ("ping-pong") variant -------------------------------------------------------------------
+// A SIMD overlaps the MFMAs of one wave with the VALU work of another only while the two are in different
+// phases, and two independent workgroups on a CU drift into the same phase.  This kernel therefore puts TWO rows
+// of the level map into one workgroup of 2*NW waves - group g = waves g*NW .. g*NW + NW - 1, wave i of either
+// group on the same SIMD - and makes the groups alternate under workgroup barriers:
+//     group 0:  M0 | V0 | M1 | V1 | ...       M_t = QK(t), then rescale + PV(t-1) with the row maximum of tile t
+//     group 1:     | M0 | V0 | M1 | ...             riding along in the shadow of its MFMAs       (matrix pipe)
+//                                             V_t = exponentials of tile t, copies of V(t+1) and K(t+2)  (VALU)
+// so the matrix phase of one group always runs next to the vector phase of the other.  The groups are otherwise
+// independent (own row, own tile buffers and schedule in LDS); rows are paired in issue order, i.e. with the
+// longest-first order neighbours of similar length, and the shorter row idles at the barriers of the longer.
+// Copies: the buffers of K(t) and V(t-1) were last read in M_t, so V(t+1) and K(t+2) are issued during V_t and
+// awaited at the start of V_(t+1), one barrier before M_(t+2) / M_(t+2) read them.
+// Only one wave per SIMD is in a given phase, so nothing else hides its latencies: the matrix phase requests its
+// operands far ahead, both phases are free of branches, and the copy instructions are spread between the
+// exponentials.
+#define PP_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+template <int D, int NW>
+__global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p) {
+  using G = psa_tiles::LtGeom<D>;
+  constexpr int F_TILE = G::TILE;
+  constexpr int NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
+  constexpr int G16 = 4 / NW;
+  constexpr int OST = D * 2 + 16;
+  static_assert(NW == 4, "4 waves per group");
+  static_assert(BM * OST <= 4 * F_TILE, "O staging must fit the tile buffers");
+  const auto P_L = p.L;
+  const auto P_bn_log2 = p.bn_log2;
+  const auto P_causal = p.causal;
+  const auto P_scale_log2 = p.scale_log2;
+  const auto P_npad = p.npad;
+  const auto P_kp = p.kp;
+  const auto P_vp = p.vp;
+  const uint32_t P_k_strb = (uint32_t)p.k_sl * 2u, P_v_strb = (uint32_t)p.v_sl * 2u;
+
+  extern __shared__ __align__(16) unsigned char smem_all[];
+  __shared__ int s_cnt[2][4], s_ioff[2][4], s_toff[2][5], s_wcnt[2][4 * NW], s_T[2];
+  const int grp = __builtin_amdgcn_readfirstlane((int)threadIdx.x / NT);
+  const int tid = (int)threadIdx.x - grp * NT, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hh = lane >> 5;
+  const uint32_t grp_base = (uint32_t)grp * (uint32_t)p.grp_bytes;
+  unsigned char* smem = smem_all + grp_base;  // this group's K buffers at 0 and F_TILE, V buffers at 2 and 3 F_TILE
+  u32x2* tdesc = (u32x2*)(smem + 4 * F_TILE);
+  uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
+
+  // pair slot of the workgroup (same dealing as the one-row kernel, in units of two rows), then this group's row
+  const int bid = blockIdx.x, sc = p.wg_chunk >> 1;
+  const int entry = ((((bid >> 3) / sc) * 8 + (bid & 7)) * sc + (bid >> 3) % sc) * 2 + grp;
+  int logical = p.order != nullptr ? p.order[entry] : entry;
+  const bool active = logical >= 0 && logical < p.total_wg;
+  if (!active) logical = 0;
+  const int I = logical % p.Mq;
+  const int bh = logical / p.Mq;
+  const int h = bh % p.Hq, b = bh / p.Hq;
+  const int hk = h / (p.Hq / p.Hkv);
+
+  int jmax = p.Nk;
+  if (P_causal) {
+    const int ce = (int)((((int64_t)(I + 1) * p.bm) + (1 << P_bn_log2) - 1) >> P_bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  if (!active) jmax = 0;
+  const int q_row0 = I * BM + wave * 32;
+  const int q_idx = q_row0 + l32;
+  bf16x8 qf[KK];
+  {
+    const int qr = q_idx < P_L ? q_idx : P_L - 1;
+    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
+  }
+  // both groups run the builder's barriers together
+  const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2, P_L,
+                                                 P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt[grp], s_ioff[grp], s_toff[grp],
+                                                 s_wcnt[grp], tid);
+  if (tid == 0) s_T[grp] = T;
+
+  const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
+  const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
+  const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
+
+  const uint32_t f_chunk = psa_tiles::lt_fetch_chunk<D>(lane);
+  uint32_t k_off[2], v_off[2];
+  psa_tiles::lt_row_operand<D>(l32, hh, k_off);
+  psa_tiles::lt_tr_operand<D>(lane, v_off);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {  // operand addresses: lane base (incl. the group's region) + immediate
+    k_off[i] += grp_base;
+    v_off[i] += grp_base;
+  }
+
+  psa_tiles::KvSource kvs;
+  kvs.k0 = kb0; kvs.v0 = vb0; kvs.kp = (const char*)P_kp; kvs.vp = (const char*)P_vp;
+  kvs.k_strb = P_k_strb; kvs.v_strb = P_v_strb;
+  kvs.BHkv = BHkv; kvs.bhk = bhk; kvs.npad = P_npad; kvs.bn_log2 = P_bn_log2; kvs.L = P_L;
+  using TileSrc = psa_tiles::TileSrc<G16>;
+  auto tile_src = [&](int t, TileSrc& a) __attribute__((always_inline)) { psa_tiles::lt_tile_src<D, G16>(kvs, tdesc, ids, t, wave, lane, a); };
+  auto issue_rows = [&](const char* base, uint32_t str, int lim, const int (&src0)[G16], int lds_byte) __attribute__((always_inline)) {
+    psa_tiles::lt_issue_rows<D, G16>(smem + lds_byte, base, str, lim, src0, wave, f_chunk);
+  };
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+
+  // ---- softmax of tile t, in pieces --------------------------------------------------------------------
+  // mask_tile: partly filled tiles and the causal diagonal (rare).  head_piece(i): piece i of the row maximum /
+  // reference update, small enough to ride along with one MFMA of PV(t-1).  prob16: the exponentials.
+  uint32_t d_cur = 0;  // descriptor word 0 of the tile whose logits are in s
+  auto mask_tile = [&](int t, f32x16 (&s_cur)[2]) __attribute__((always_inline)) {
+    const uint32_t d = d_cur;
+    const int lv = d & 3;
+    const int nvalid = (int)((d >> 3) & 127);
+    const int qlim = (q_idx + 1) >> lv;
+    const uint32_t d1 = __builtin_amdgcn_readfirstlane(tdesc[t][1]);
+    const int cnt = (int)(d1 >> 16), lt = (int)(d >> 10), sbs_log2 = P_bn_log2 - lv;
+    const uint16_t* lids = ids + (d1 & 0xffff);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int r0 = c * 32 + g * 8 + hh * 4;
+        int keep = nvalid - r0;
+        if (P_causal) {
+          const int gpos = (lt << 6) + r0;
+          int bi = gpos >> sbs_log2;
+          bi = bi < cnt - 1 ? bi : cnt - 1;
+          const int src0 = ((int)lids[bi] << sbs_log2) + (gpos & ((1 << sbs_log2) - 1));
+          keep = keep < qlim - src0 ? keep : qlim - src0;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s_cur[c][g * 4 + e] = e < keep ? s_cur[c][g * 4 + e] : -INFINITY;
+      }
+  };
+  constexpr int HEAD_PIECES = 12;
+  float hx0, hx1, h_cand, h_new;  // state between the pieces
+  float alpha = 1.0f, nb = 0.f;
+  auto head_piece = [&](int i, const f32x16 (&s_cur)[2], bool real) __attribute__((always_inline)) {
+    if (i == 0) {
+      hx0 = s_cur[0][0];
+      hx1 = s_cur[1][0];
+    }
+    if (i < 7) {
+      hx0 = max3f(hx0, s_cur[0][1 + 2 * i], s_cur[0][2 + 2 * i]);
+      hx1 = max3f(hx1, s_cur[1][1 + 2 * i], s_cur[1][2 + 2 * i]);
+    } else if (i == 7) {
+      hx0 = max3f(hx0, s_cur[0][15], fmaxf(hx1, s_cur[1][15]));
+    } else if (i == 8) {
+      hx0 = half_wave_max(hx0);
+    } else if (i == 9) {
+      h_cand = __builtin_fmaf(hx0, P_scale_log2, (float)(d_cur & 3));
+    } else if (i == 10) {
+      // raise the reference max only when it lags by more than the threshold (or is still -inf)
+      h_new = (h_cand - m_run > LAZY_THRESHOLD) ? h_cand : m_run;
+      h_new = (m_run == -INFINITY) ? h_cand : h_new;
+    } else if (i == 11) {
+      const float m_use = h_new == -INFINITY ? 0.f : h_new;  // rows that still see no key
+      alpha = real ? fast_exp2(m_run - m_use) : 1.0f;
+      nb = (float)(d_cur & 3) - m_use;
+      m_run = real ? h_new : m_run;
+    }
+  };
+  // probabilities of 4 logits: exp2, round to bf16 for P^T; the row sum adds the unrounded values with plain adds
+  // (a dot-product instruction would queue behind the other group's MFMAs)
+  auto prob4 = [&](const f32x16& sc, int i, float nb_, uint32_t* pk2, float& lsum) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 4; e += 2) {
+      const float p0 = fast_exp2(__builtin_fmaf(sc[i + e], P_scale_log2, nb_));
+      const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb_));
+      pk2[e >> 1] = pack_bf16x2(p0, p1);
+      lsum += p0 + p1;
+    }
+  };
+  // Copy source of a tile for this lane: base pointers and row strides of its level (uniform), and the RPL
+  // consecutive source rows of this wave's 16-row group (clamped where a partly filled tile runs past the end).
+  struct CopySrc {
+    const char *kbase, *vbase;
+    uint32_t kstr, vstr;
+    int row[G::RPL];
+  };
+  // base pointers of the pooled levels of this (batch, kv head); plain scalars, selected by compare chains
+  auto pool_base = [&](const bf16_t* pool, int lv) __attribute__((always_inline)) {
+    return (const char*)pool + (BHkv * (P_npad - (P_npad >> (lv - 1))) + bhk * (P_npad >> lv)) * (D * 2);
+  };
+  const char* const kb1 = pool_base(P_kp, 1);
+  const char* const kb2 = pool_base(P_kp, 2);
+  const char* const kb3 = pool_base(P_kp, 3);
+  const char* const vb1 = pool_base(P_vp, 1);
+  const char* const vb2 = pool_base(P_vp, 2);
+  const char* const vb3 = pool_base(P_vp, 3);
+  auto by_level = [&](int lv, const char* a0, const char* a1, const char* a2, const char* a3) __attribute__((always_inline)) {
+    const char* r = a0;
+    r = lv == 1 ? a1 : r;
+    r = lv == 2 ? a2 : r;
+    r = lv == 3 ? a3 : r;
+    return r;
+  };
+  // One copy instruction: block n of this wave's 16-row group, into the tile buffer at byte lds_byte of the group
+  auto issue_one = [&](const char* base, uint32_t str, int row, int lds_byte, int n) __attribute__((always_inline)) {
+    psa_tiles::lds_copy16(base, __umul24((uint32_t)row, str) + f_chunk, psa_tiles::lds_addr_of(smem + lds_byte + (wave * G::RPL + n) * F_ISTR));
+  };
+  // The matrix work of one phase: S^T = K Q^T (tile in K buffer KB) and then O^T += V^T P^T (tile in V buffer
+  // 1 - KB, probabilities pk2).  Only one wave per SIMD is in its matrix phase, so nothing else hides the LDS
+  // latency: all 2*KK K operands are requested up front, and the V^T operands follow into the registers that
+  // the QK steps release (two PV steps per k-step), so that the MFMAs stream.  hook(st) runs after PV step st.
+  static_assert(4 * DB == 2 * KK, "two PV steps per QK k-step");
+  auto matrix_work = [&](auto kb_c, f32x16 (&s2)[2], const uint32_t (&pk2)[2][8], float a_prev, auto mid, auto hook) __attribute__((always_inline)) {
+    constexpr int KB = decltype(kb_c)::value;
+    constexpr int STEPS = 4 * DB;
+    PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem_all) + KB * F_TILE;
+    PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem_all) + (2 + (KB ^ 1)) * F_TILE;
+    constexpr int K_UP = KK - 2;          // k-steps whose K operands are requested before the first MFMA
+    constexpr int V_LATE = 2 * (KK - K_UP);  // PV steps whose operands are requested during PV
+    bf16x8 ka[2 * KK];
+    auto kread = [&](int kk) __attribute__((always_inline)) {
+      ka[2 * kk] = *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64);
+      ka[2 * kk + 1] = *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + G::HALF);
+    };
+#pragma unroll
+    for (int kk = 0; kk < K_UP; ++kk) kread(kk);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s2[c][i] = 0.f;
+    u32x2 vlo[STEPS], vhi[STEPS];
+    auto vread = [&](int st) __attribute__((always_inline)) {
+      const int cg = st / DB, db = st % DB;
+      const int off = (cg >> 1) * G::HALF + db * 64 + (cg & 1) * G::GROUP;
+      vlo[st] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0] + off)));
+      vhi[st] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1] + off)));
+    };
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      s2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[2 * kk], qf[kk], s2[0], 0, 0, 0);
+      s2[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[2 * kk + 1], qf[kk], s2[1], 0, 0, 0);
+      if (kk + K_UP < KK) {
+        kread(kk + K_UP);
+      } else {
+        vread(2 * (kk - (KK - K_UP)));
+        vread(2 * (kk - (KK - K_UP)) + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mid();
+    if (__any(a_prev != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] *= a_prev;
+    }
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const int cg = st / DB, db = st % DB;
+      const uint32_t* pk8 = pk2[cg >> 1];
+      const int g = cg & 1;
+      u32x4 bw = {pk8[g * 4 + 0], pk8[g * 4 + 1], pk8[g * 4 + 2], pk8[g * 4 + 3]};
+      u32x4 aw = {vlo[st][0], vlo[st][1], vhi[st][0], vhi[st][1]};
+      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), __builtin_bit_cast(bf16x8, bw), acc[db], 0, 0, 0);
+      if (st < V_LATE) vread(STEPS - V_LATE + st);
+      hook(st);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  const std::integral_constant<int, 0> B0;
+  const std::integral_constant<int, 1> B1;
+
+  CopySrc ts, ts2;
+  f32x16 s[2];
+  uint32_t pk[2][8];
+  auto to_copy_src = [&](const TileSrc& a, CopySrc& c) __attribute__((always_inline)) {
+    c.kbase = a.kbase; c.vbase = a.vbase; c.kstr = a.kstr; c.vstr = a.vstr;
+#pragma unroll
+    for (int n = 0; n < G::RPL; ++n) c.row[n] = a.src0[0] + n < a.lim ? a.src0[0] + n : a.lim;
+  };
+  // first copies: K(0), V(0), K(1); ts is left describing tile min(1, T-1) for the copy of V(1)
+  if (T > 0) {
+    TileSrc a;
+    tile_src(0, a);
+    issue_rows(a.kbase, a.kstr, a.lim, a.src0, 0);
+    issue_rows(a.vbase, a.vstr, a.lim, a.src0, 2 * F_TILE);
+    if (T > 1) {
+      tile_src(1, a);
+      issue_rows(a.kbase, a.kstr, a.lim, a.src0, F_TILE);
+    }
+    to_copy_src(a, ts);
+  } else {
+    ts.kbase = kb0; ts.vbase = vb0; ts.kstr = 0; ts.vstr = 0;
+#pragma unroll
+    for (int n = 0; n < G::RPL; ++n) ts.row[n] = 0;
+  }
+  ts2 = ts;
+  // M_0 multiplies V buffer 1 by zero probabilities: give it finite contents
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) pk[c][i] = 0u;
+  for (int u = tid * 16; u < F_TILE; u += NT * 16) *(u32x4*)(smem + 3 * F_TILE + u) = u32x4{0u, 0u, 0u, 0u};
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+  const int T_other = s_T[grp ^ 1];
+  const int C = (T > T_other ? T : T_other) + 1;  // (M, V) phase pairs both groups step through
+
+  // M_t: the matrix phase.  K(t) lives in K buffer t&1, V(t-1) in V buffer (t-1)&1.  QK(t) comes first so that
+  // the row maximum of tile t can ride along with the MFMAs of PV(t-1), and so does the look-up of the source
+  // rows of tile t+2 (two dependent LDS reads, spread over the phase).  At t == T only PV(T-1) counts: QK then
+  // runs on stale data and its maximum is dropped; at t == 0 PV multiplies the zeroed V buffer by zeros.
+  // Both phases are free of branches (tiles past the end are clamped to the last one and copied again into a
+  // buffer nobody reads), so that the instruction order below is the order that runs.
+  constexpr int HOOK0 = 2;  // first PV step that carries a piece of the maximum (QK's last results need that long)
+  const int T_last = T > 0 ? T - 1 : 0;
+  uint32_t d_next = T > 0 ? __builtin_amdgcn_readfirstlane(tdesc[0][0]) : 0u;  // descriptor of the tile of the next M phase
+  auto mfma_phase = [&](int t, auto cur_c) __attribute__((always_inline)) {
+    if (T > 0 && t <= T) {
+      const bool real = t < T;
+      d_cur = real ? d_next : 0u;
+      matrix_work(
+          cur_c, s, pk, alpha,
+          [&]() __attribute__((always_inline)) {
+            if (d_cur & 4) mask_tile(t, s);
+          },
+          [&](int st) __attribute__((always_inline)) {
+            if (st >= HOOK0 && st - HOOK0 < HEAD_PIECES) head_piece(st - HOOK0, s, real);
+          });
+    }
+  };
+  // V_t: the vector phase.  K buffer t&1 and V buffer (t-1)&1 were last read in M_t: V(t+1) (described by ts) and
+  // K(t+2) (ts2, looked up in the first half of this phase) go there, one copy instruction per 4 exponentials so
+  // that the copy unit never makes the wave wait.
+  auto valu_phase = [&](int t, auto cur_c) __attribute__((always_inline)) {
+    constexpr int CUR = decltype(cur_c)::value;
+    if (t < T) {
+      const int tn = t + 2 < T ? t + 2 : T_last;
+      const u32x2 dd2 = tdesc[tn];
+      const uint32_t dn = tdesc[t + 1 < T ? t + 1 : T_last][0];
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1), V(t) of this wave have landed (visible to the group after the next barrier)
+      float lsum = 0.f;
+      int n_lv = 0, n_sbs = 0, n_g = 0, n_lim = 0;
+      uint16_t n_id = 0;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (c < 4) issue_one(ts.vbase, ts.vstr, ts.row[c], (2 + (CUR ^ 1)) * F_TILE, c);
+        else issue_one(ts2.kbase, ts2.kstr, ts2.row[c - 4], CUR * F_TILE, c - 4);
+        prob4(s[c >> 2], (c & 3) * 4, nb, pk[c >> 2] + (c & 3) * 2, lsum);
+        if (c == 0) {
+          const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd2[0]), d1 = __builtin_amdgcn_readfirstlane(dd2[1]);
+          d_next = __builtin_amdgcn_readfirstlane(dn);
+          n_lv = d0 & 3;
+          const int nvalid = (d0 >> 3) & 127, lt = d0 >> 10, cnt = d1 >> 16;
+          n_sbs = P_bn_log2 - n_lv;
+          n_lim = (nvalid < TK && n_lv == 0) ? P_L - 1 : 0x7fffffff;
+          n_g = (lt << 6) + wave * 16 + psa_tiles::lt_fetch_row<D>(lane);
+          int bi = n_g >> n_sbs;
+          bi = bi < cnt - 1 ? bi : cnt - 1;  // (only matters in a partly filled tile)
+          n_id = ids[(d1 & 0xffff) + bi];
+        }
+        if (c == 2) {
+          ts2.kbase = by_level(n_lv, kb0, kb1, kb2, kb3);
+          ts2.vbase = by_level(n_lv, vb0, vb1, vb2, vb3);
+          ts2.kstr = n_lv == 0 ? P_k_strb : (uint32_t)(D * 2);
+          ts2.vstr = n_lv == 0 ? P_v_strb : (uint32_t)(D * 2);
+        }
+        if (c == 3) {
+          const int src0 = ((int)n_id << n_sbs) + (n_g & ((1 << n_sbs) - 1));
+#pragma unroll
+          for (int n = 0; n < G::RPL; ++n) ts2.row[n] = src0 + n < n_lim ? src0 + n : n_lim;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      ts = ts2;
+      l_run = l_run * alpha + lsum;
+    }
+  };
+  if (grp == 1) PP_BARRIER();
+  for (int t = 0; t < C; t += 2) {
+    mfma_phase(t, B0);
+    PP_BARRIER();
+    valu_phase(t, B0);
+    PP_BARRIER();
+    mfma_phase(t + 1, B1);
+    PP_BARRIER();
+    valu_phase(t + 1, B1);
+    PP_BARRIER();
+  }
+  if (grp == 0) PP_BARRIER();
+
+  // ---- epilogue ---------------------------------------------------------------------------------------
+  float l_tot = half_wave_sum(l_run);
+  const float l_safe = fmaxf(l_tot, 1e-8f);
+  const float inv = 1.0f / l_safe;
+  if (active && p.lse != nullptr && hh == 0 && q_idx < P_L) {
+    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // the last (repeated) tile copies land in the buffers that now stage O
+  __syncthreads();
+  unsigned char* Os = smem;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
+      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
+      *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
+    }
+  __syncthreads();
+  if (active) {
+    bf16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
+    for (int u = tid; u < BM * CH; u += NT) {
+      const int r = u / CH, ch = u % CH;
+      const int row = I * BM + r;
+      if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+    }
+  }
+}
+
 // ---- longest-rows-first ordering ---------------------------------------------------------------------
 // Rows of the level map differ in the number of tiles they retain.  Workgroup ids are dealt round-robin
 // to the 8 XCDs and each XCD runs its ids in order, so sorting every XCD's share by decreasing tile count
@@ -420,12 +846,29 @@ int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   return PSA_OK;
 }
 
+template <int D, int NW>
+int launch_fwd_pp(FwdParams& p, int Nk, hipStream_t stream) {
+  const size_t sched = (((size_t)p.max_tiles * 8 + (size_t)Nk * 2) + 15) & ~(size_t)15;
+  p.grp_bytes = (int)(4 * psa_tiles::LtGeom<D>::TILE + sched);
+  const size_t shmem = 2 * (size_t)p.grp_bytes;
+  if (hipFuncSetAttribute((const void*)psa_fwd_pp_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+    return PSA_ERR_LAUNCH;
+  hipLaunchKernelGGL((psa_fwd_pp_kernel<D, NW>), dim3((unsigned)((p.wg_chunk / 2) * p.wg_groups)), dim3(2 * NW * 64), shmem, stream, p);
+  return PSA_OK;
+}
+// LDS bytes the two-group kernel needs (tile buffers and schedule of both groups + its static tables)
+template <int D>
+size_t pp_lds_bytes(int max_tiles, int Nk) {
+  const size_t sched = (((size_t)max_tiles * 8 + (size_t)Nk * 2) + 15) & ~(size_t)15;
+  return 2 * (4 * (size_t)psa_tiles::LtGeom<D>::TILE + sched) + 512;
+}
+
 }  // namespace
 
 extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
   if (B <= 0 || Hq <= 0 || L <= 0 || block_m <= 0) return 0;
   const int64_t total = (int64_t)B * Hq * ((L + block_m - 1) / block_m);
-  return 2 * (total + 8 * FWD_MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
+  return 2 * (total + 16 * FWD_MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
 }
 
 extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
@@ -477,6 +920,10 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.wg_chunk = (int)((total + p.wg_groups - 1) / p.wg_groups);
   // worst case: every kv-block at level 1, plus one partly filled tile per pooled level
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
+  p.grp_bytes = 0;
+  // two rows per workgroup when the head dim / block size have that kernel and both schedules fit into LDS
+  const bool two_group = D == 128 && block_m == 128 && total > 1 && pp_lds_bytes<128>(p.max_tiles, Nk) <= 160 * 1024 && !PSA_FWD_ONE_GROUP;
+  if (two_group) p.wg_chunk = (p.wg_chunk + 1) & ~1;  // pairs never straddle two groups of rows
   p.order = nullptr;
   if (workspace != nullptr && map != nullptr && total > 8 * 32) {
     PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
@@ -490,7 +937,8 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     p.order = order;
   }
   int rc;
-  if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
+  if (two_group) rc = launch_fwd_pp<128, 4>(p, Nk, (hipStream_t)stream);
+  else if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
   else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);
   else if (block_m == 128) rc = launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
   else rc = launch_fwd<64, 2>(p, Nk, (hipStream_t)stream);

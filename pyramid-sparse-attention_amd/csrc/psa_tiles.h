@@ -41,9 +41,9 @@ struct RowSchedule {
 template <int NT>
 __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem, int64_t mrow, int Nk, int jmax, int bn_log2,
                                                   int L, bool causal, int64_t q_first_row, uint16_t* ids, u32x2* tdesc,
-                                                  int* s_cnt, int* s_ioff, int* s_toff, int* s_wcnt) {
+                                                  int* s_cnt, int* s_ioff, int* s_toff, int* s_wcnt, int tid) {
   constexpr int NW = NT / 64;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = tid >> 6;
   // wave w owns columns [w * share, min(jmax, (w + 1) * share)), share a multiple of 64
   const int share = ((jmax + 64 * NW - 1) / (64 * NW)) * 64;
   const int j_lo = wave * share, j_hi = (wave + 1) * share < jmax ? (wave + 1) * share : jmax;
@@ -132,6 +132,14 @@ __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem,
   }
   __syncthreads();
   return T;
+}
+
+template <int NT>
+__device__ __forceinline__ int build_row_schedule(const void* map, int map_elem, int64_t mrow, int Nk, int jmax, int bn_log2,
+                                                  int L, bool causal, int64_t q_first_row, uint16_t* ids, u32x2* tdesc,
+                                                  int* s_cnt, int* s_ioff, int* s_toff, int* s_wcnt) {
+  return build_row_schedule<NT>(map, map_elem, mrow, Nk, jmax, bn_log2, L, causal, q_first_row, ids, tdesc, s_cnt, s_ioff,
+                                s_toff, s_wcnt, (int)threadIdx.x);
 }
 
 struct TileRef {
@@ -290,6 +298,16 @@ __device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tde
   }
 }
 
+// One global -> LDS copy instruction: lane l's 16 bytes at sbase + voff(l) land at LDS address lds_addr + 16 * l.
+// sbase and lds_addr are wave-uniform.  Written as inline assembly on purpose: the compiler then does not know
+// that a copy into LDS is in flight and so does not put a vmcnt(0) wait in front of every LDS read it cannot
+// tell apart from the copy's target (it cannot for the transposing reads).  The kernels wait (vmcnt) and
+// synchronise explicitly before a tile is read.
+__device__ __forceinline__ void lds_copy16(const char* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(PSA_LDS(const void))(p); }
+
 // Copies this wave's groups of one tile: one block per instruction goes to block RPL*g16 + n of the tile at `dst`.
 template <int D, int G16>
 __device__ __forceinline__ void lt_issue_rows(unsigned char* dst, const char* base, uint32_t str, int lim, const int (&src0)[G16],
@@ -302,13 +320,12 @@ __device__ __forceinline__ void lt_issue_rows(unsigned char* dst, const char* ba
       // the usual case: the uniform base pointer steps from row to row, the lane offset stays
       const uint32_t off = (uint32_t)src0[gi] * str + f_chunk;
 #pragma unroll
-      for (int n = 0; n < G::RPL; ++n)
-        __builtin_amdgcn_global_load_lds(base + (uint64_t)(n * str) + off, (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
+      for (int n = 0; n < G::RPL; ++n) lds_copy16(base + (uint64_t)(n * str), off, lds_addr_of(dst + (blk + n) * LT_ISTR));
     } else {
 #pragma unroll
       for (int n = 0; n < G::RPL; ++n) {
         const int src = src0[gi] + n < lim ? src0[gi] + n : lim;
-        __builtin_amdgcn_global_load_lds(base + ((uint32_t)src * str + f_chunk), (PSA_LDS(void))(dst + (blk + n) * LT_ISTR), 16, 0, 0);
+        lds_copy16(base, (uint32_t)src * str + f_chunk, lds_addr_of(dst + (blk + n) * LT_ISTR));
       }
     }
   }
