@@ -303,8 +303,20 @@ __device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tde
 // that a copy into LDS is in flight and so does not put a vmcnt(0) wait in front of every LDS read it cannot
 // tell apart from the copy's target (it cannot for the transposing reads).  The kernels wait (vmcnt) and
 // synchronise explicitly before a tile is read.
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {  // tells the compiler the value is wave-uniform
+  const uint64_t a = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ void lds_copy16(const char* sbase, uint32_t voff, uint32_t lds_addr) {
+  sbase = uniform_ptr(sbase);
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+// the same with a full per-lane address
+__device__ __forceinline__ void lds_copy16_addr(const char* vaddr, uint32_t lds_addr) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(vaddr) : "memory");
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(PSA_LDS(const void))(p); }
 
