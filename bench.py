@@ -46,8 +46,8 @@ WORKLOADS.update({
 WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
 
 
-# psa_fwd_lds_kernel<128, 4> at workload c2: (1080692.5 * 2.000 + 98280.0) KiB per dispatch
-FWD_TRAFFIC_BYTES = {"c2": 2.314e9}
+# psa_fwd_pp_kernel<128, 4> at workload c2: (850380.5 * 2.000 + 98280.0) KiB per dispatch
+FWD_TRAFFIC_BYTES = {"c2": 1.842e9}
 
 
 def scaled_ratios(tau):
@@ -151,7 +151,7 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
         "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
                    "sparsity": round(1 - density, 4)},
         "stages_ms": stages,
-        "roofline": {"kernel": "psa_fwd_lds_kernel", "bound": "mfma",
+        "roofline": {"kernel": "psa_fwd_pp_kernel", "bound": "mfma",
                      "achieved": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "flops_per_launch": fwd_flops, "avg_launch_ms": round(t_fwd_avg, 4)},
@@ -259,7 +259,7 @@ def main():
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
 
     roofline = {
-        "kernel": "psa_fwd_lds_kernel",
+        "kernel": "psa_fwd_pp_kernel",
         "bound": "mfma",
         "achieved": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12, 2),
         "peak": PEAK_BF16_TFLOPS,
