@@ -77,6 +77,36 @@ def test_fwd_odd_counts_of_small_blocks():
         run_case(1, 1, 1, L, 64, 128, 128, False, seed=n8, lmap=mm)
 
 
+def test_fwd_two_row_workgroups_uneven_rows():
+    # head dim 128 with 128-row q-blocks runs two map rows per workgroup: pair rows of very different length
+    # (many tiles / one partly filled tile / none), an odd number of rows, partly filled level-4/8 tiles
+    L = 1024 - 37
+    for causal in (False, True):
+        mm = np.zeros((1, 3, 8, 8), np.int32)
+        mm[0, 0, 0, :] = 1            # 16 tiles next to ...
+        mm[0, 0, 1, 0] = 8            # ... a quarter of a tile
+        mm[0, 0, 3, :3] = 8           # empty row 2 next to 3/4 of a tile
+        mm[0, 0, 4, :] = 2
+        mm[0, 0, 5, 1:4] = 4
+        mm[0, 0, 7, :] = [1, 2, 4, 8, 8, 4, 2, 1]
+        mm[0, 1] = 1
+        mm[0, 2, 5:, :] = 4           # head 2: rows 0-4 empty
+        if causal:
+            mm = np.where(np.arange(8)[None, None, None, :] > np.arange(8)[None, None, :, None], 0, mm)
+        for balance in (True, False):
+            from psa_hip import ops
+
+            q, k, v = rnd(1, 3, L, 128, seed=5), rnd(1, 3, L, 128, seed=6), rnd(1, 3, L, 128, seed=7)
+            out, lse, _ = ops.sparse_attention_fwd(q.to(dev()), k.to(dev()), v.to(dev()), torch.from_numpy(mm).to(dev()), 128, 128,
+                                                  causal=causal, return_lse=True, balance=balance)
+            ref, ref_lse = O.psa_attention_dense(q, k, v, mm, 128, 128, causal=causal)
+            mx, mean = attn_errors(out, ref)
+            assert mx <= MAX_ABS and mean <= MEAN_ABS, (causal, balance, mx, mean)
+            fin = torch.isfinite(ref_lse)
+            assert torch.equal(torch.isfinite(lse.cpu()), fin)
+            assert float((lse.cpu().double()[fin] - ref_lse[fin]).abs().max()) <= 2e-2
+
+
 def test_fwd_dense_equals_sdpa_and_all_ones_map():
     from psa_hip import ops
 
