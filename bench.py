@@ -21,6 +21,7 @@ sys.path.insert(0, PKG)
 
 METRIC = "PSA attn ms/layer + effective TFLOPS (% bf16 MFMA peak) at Wan2.1-1.3B shape, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+SUSTAINED_BF16_TFLOPS = 1800.0  # measured: pure MFMA loop, random bf16 operands, 30-60 ms, one MI355X
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
@@ -271,6 +272,10 @@ def main():
         "flops_per_launch": exec_flops,
         "avg_launch_ms": round(t_fwd_avg, 4),
         "launch_includes": "the forward kernel and its two row-ordering launches (about 9 us together)",
+        # a register-only loop of independent bf16 MFMAs with random operands sustains this much on the same chip
+        # (power management); with constant operands it reaches 2460
+        "sustained_mfma_tflops_random_operands": SUSTAINED_BF16_TFLOPS,
+        "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / SUSTAINED_BF16_TFLOPS, 4),
     }
 
     # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------

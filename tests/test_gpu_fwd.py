@@ -126,6 +126,28 @@ def test_fwd_dense_equals_sdpa_and_all_ones_map():
     assert mx <= MAX_ABS and mean <= MEAN_ABS
 
 
+def test_fwd_long_sequence_takes_the_one_row_kernel():
+    # with 128-key blocks the schedules of two rows stop fitting into LDS above ~85k tokens: the launch falls back
+    # to one row per workgroup.  Dense attention on 88k tokens against torch SDPA on the GPU (bf16), plus a sparse
+    # map through the size-independent property that rows whose blocks are all level 1 equal the dense rows.
+    from psa_hip import ops
+
+    B, H, L, D = 1, 1, 88000, 128
+    g = torch.Generator(device="cpu").manual_seed(11)
+    q, k, v = (torch.randn(B, H, L, D, generator=g).to(torch.bfloat16).to(dev()) for _ in range(3))
+    ref = F.scaled_dot_product_attention(q, k, v).float()
+    o = ops.sparse_attention_fwd(q, k, v, None, 128, 128)
+    assert float((o.float() - ref).abs().max()) <= MAX_ABS and float((o.float() - ref).abs().mean()) <= MEAN_ABS
+    Nk = -(-L // 128)
+    mp = torch.zeros(B, H, Nk, Nk, dtype=torch.int8, device=dev())
+    mp[..., ::7, :] = 1          # every 7th q-block keeps everything at level 1
+    mp[..., 1::7, ::3] = 4       # some other rows: a third of the blocks, pooled 4x
+    o2 = ops.sparse_attention_fwd(q, k, v, mp, 128, 128)
+    rows = torch.arange(L, device=dev()) // 128 % 7 == 0
+    assert float((o2[..., rows, :].float() - ref[..., rows, :]).abs().max()) <= MAX_ABS
+    assert torch.isfinite(o2.float()).all()
+
+
 def test_fwd_lossless_pooling_invariant_full_size_heads():
     """K and V constant inside aligned groups of 8 tokens: every map without skips must give plain
     attention - checked at the Wan2.1-1.3B sequence length on one head against SDPA on the GPU."""
