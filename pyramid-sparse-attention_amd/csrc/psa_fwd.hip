@@ -20,9 +20,11 @@
 //    ONE query column: the softmax row max / row sum are in-lane reductions plus a single exchange between the
 //    two half-waves (v_permlane32_swap), and P^T is already in B-operand layout.
 //  * Online softmax in base 2: p = exp2(s*scale*log2e + log2(level) - m); the reference maximum is only raised
-//    when it lags by more than 2^8 (lazy rescaling), so most tiles skip the accumulator rescale.  Row sums add
-//    the bf16-ROUNDED probabilities (v_dot2_f32_bf16): numerator and denominator use the same values.
-//  * One barrier per tile: copy of tile t+1 in flight | QK(t) | softmax(t) | PV(t) | barrier.
+//    when it lags by more than 2^8 (lazy rescaling), so most tiles skip the accumulator rescale.  Row sums: the
+//    one-row kernel adds the bf16-ROUNDED probabilities (v_dot2_f32_bf16: numerator and denominator use the same
+//    values), the two-row kernel the unrounded ones with plain adds as the reference does (a dot-product
+//    instruction runs on the matrix pipe and would queue behind the other group's MFMAs).
+//  * One-row kernel: one barrier per tile: copy of tile t+1 in flight | QK(t) | softmax(t) | PV(t) | barrier.
 //  * Rows are issued in groups (group g on XCD g mod 8, a few heads per phase of 8 groups) and, with the
 //    optional workspace, longest first inside a group.
 //
