@@ -152,7 +152,7 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
         "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
                    "sparsity": round(1 - density, 4)},
         "stages_ms": stages,
-        "roofline": {"kernel": "psa_fwd_pp_kernel", "bound": "mfma",
+        "roofline": {"kernel": "psa_fwd_pp_kernel" if (D == 128 and bm == 128) else "psa_fwd_lds_kernel", "bound": "mfma",
                      "achieved": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "flops_per_launch": fwd_flops, "avg_launch_ms": round(t_fwd_avg, 4)},
@@ -260,7 +260,7 @@ def main():
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
 
     roofline = {
-        "kernel": "psa_fwd_pp_kernel",
+        "kernel": "psa_fwd_pp_kernel" if (D == 128 and bm == 128) else "psa_fwd_lds_kernel",
         "bound": "mfma",
         "achieved": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12, 2),
         "peak": PEAK_BF16_TFLOPS,
