@@ -144,6 +144,15 @@ int psa_ksim(psa_tensor4 k, int32_t* cap_out, int B, int H, int L, int D, int bl
 int psa_map_min_cap(void* map, int map_elem_bytes, const int32_t* cap, int64_t bh, int Mq, int Nk,
                     psa_stream_t stream);
 
+/* Token re-ordering: dst[t][b, h, i, :] = src[t][b, h, index[i], :] for i < L_dst, for n_tensors (1..3) tensors
+ * that share the index vector (q, k, v in one launch; heads[t] heads each).  index: int32 [L_dst], values in
+ * [0, L_src).  Rows are D elements of elem_bytes (2 or 4) bytes; strides are in elements.
+ * Replaces the index_select + cat of GilbertRearranger.rearrange / reversed_rearrange:
+ * reference src/psa_triton/utils/rearranger.py:14-132. */
+int psa_gather_rows(const psa_tensor4* src, const psa_tensor4* dst, const int* heads, int n_tensors,
+                    const int32_t* index, int B, int L_dst, int L_src, int D, int elem_bytes,
+                    psa_stream_t stream);
+
 /* mean(1/level) over the map, skipped blocks counting 0; causal != 0 counts lower-triangle pairs only.
  * density_out: one float per (b, h) row of the [BH] vector, plus the overall mean at index BH.
  * reference src/psa_triton/utils/transfer_attn_to_mask.py:510-544. */

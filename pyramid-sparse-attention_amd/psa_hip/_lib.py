@@ -55,6 +55,8 @@ SIGNATURES = {
     "psa_ksim": (c_int, [Tensor4, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p]),
     "psa_map_min_cap": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "psa_density": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "psa_gather_rows": (c_int, [POINTER(Tensor4), POINTER(Tensor4), POINTER(c_int), c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                c_void_p]),
     "psa_fwd": (
         c_int,
         [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,

@@ -204,6 +204,34 @@ def estimate_xattn(q: torch.Tensor, k: torch.Tensor, block_size: int = 128, stri
     return est
 
 
+def gather_rows(tensors: Sequence[torch.Tensor], index: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+    """out[t][b, h, i, :] = tensors[t][b, h, index[i], :] for up to three [B, H, L, D] tensors of one dtype
+    (2- or 4-byte elements, D contiguous) that share the int32 index vector: the token re-ordering of
+    GilbertRearranger (reference utils/rearranger.py:14-132) in one launch instead of index_select + cat per tensor."""
+    _require_gpu(*tensors, index)
+    if not 1 <= len(tensors) <= 3:
+        raise ValueError("gather_rows takes 1 to 3 tensors")
+    t0 = tensors[0]
+    B, _, L_src, D = t0.shape
+    for t in tensors:
+        if t.dim() != 4 or t.dtype != t0.dtype or t.shape[0] != B or t.shape[2] != L_src or t.shape[3] != D:
+            raise ValueError("tensors must be [B, H, L, D] with the same dtype, B, L and D")
+    if index.dtype != torch.int32 or index.dim() != 1:
+        raise ValueError("index must be a 1-D int32 tensor")
+    index = index.contiguous()
+    srcs = [t if t.stride(3) == 1 else t.contiguous() for t in tensors]
+    L_dst = index.numel()
+    outs = [torch.empty(B, t.shape[1], L_dst, D, dtype=t.dtype, device=t.device) for t in srcs]
+    n = len(srcs)
+    a_src = (Tensor4 * 3)(*[_t4(t) for t in srcs], *[_t4(srcs[0])] * (3 - n))
+    a_dst = (Tensor4 * 3)(*[_t4(t) for t in outs], *[_t4(outs[0])] * (3 - n))
+    heads = (ctypes.c_int * 3)(*[t.shape[1] for t in srcs], *[srcs[0].shape[1]] * (3 - n))
+    with torch.cuda.device(t0.device):
+        check(lib.psa_gather_rows(a_src, a_dst, heads, n, _ptr(index), B, L_dst, L_src, D, t0.element_size(), _stream(t0)),
+              "psa_gather_rows")
+    return tuple(outs)
+
+
 def map_from_list(list_mask: torch.Tensor, Nk: int, map_dtype: torch.dtype = torch.int8) -> torch.Tensor:
     """Index list [..., W] int32 -> dense level map [..., Nk]."""
     _require_gpu(list_mask)

@@ -33,7 +33,34 @@ class GilbertRearranger:
             self._cache[key] = src.to(device)
         return self._cache[key]
 
+    def _combined_index(self, device, forward: bool) -> torch.Tensor:
+        """int32 [L] source row of every output row, text tokens included: forward moves the text (first
+        text_length rows) behind the re-ordered video tokens, backward moves it to the front again."""
+        key = (str(device), forward, "combined")
+        if key not in self._cache:
+            t, n = self.text_length, self.total_elements
+            if forward:
+                idx = torch.cat((self.original_order2gilbert_order_cpu + t, torch.arange(t)))
+            else:
+                idx = torch.cat((torch.arange(t) + n, self.gilbert_order2original_order_cpu))
+            self._cache[key] = idx.to(torch.int32).to(device)
+        return self._cache[key]
+
+    @staticmethod
+    def _native(x: torch.Tensor) -> bool:
+        # the HIP row gather handles GPU tensors [B, H, L, D] with 2- or 4-byte elements and 16-byte rows
+        return (x.is_cuda and x.dim() == 4 and x.element_size() in (2, 4) and (x.shape[-1] * x.element_size()) % 16 == 0
+                and 256 % ((x.shape[-1] * x.element_size()) // 16) == 0 and x.data_ptr() % 16 == 0
+                and all((s * x.element_size()) % 16 == 0 for s in x.stride()[:3]))
+
     def rearrange_single(self, x: torch.Tensor) -> torch.Tensor:
+        if self._native(x) and x.shape[-2] == self.total_elements + self.text_length:
+            from .. import ops
+
+            return ops.gather_rows((x,), self._combined_index(x.device, True))[0]
+        return self._rearrange_single_torch(x)
+
+    def _rearrange_single_torch(self, x: torch.Tensor) -> torch.Tensor:
         idx = self._indices(x.device, True)
         if self.text_length == 0:
             return x.index_select(-2, idx)
@@ -41,9 +68,22 @@ class GilbertRearranger:
         return torch.cat((video.index_select(-2, idx), text), dim=-2)
 
     def rearrange(self, q, k, v) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        L = self.total_elements + self.text_length
+        if (all(self._native(t) and t.shape[-2] == L for t in (q, k, v)) and q.dtype == k.dtype == v.dtype
+                and q.shape[0] == k.shape[0] == v.shape[0] and q.shape[-1] == k.shape[-1] == v.shape[-1]):
+            from .. import ops
+
+            return ops.gather_rows((q, k, v), self._combined_index(q.device, True))  # one launch for the three
         return self.rearrange_single(q), self.rearrange_single(k), self.rearrange_single(v)
 
     def reversed_rearrange(self, out: torch.Tensor) -> torch.Tensor:
+        if self._native(out) and out.shape[-2] == self.total_elements + self.text_length:
+            from .. import ops
+
+            return ops.gather_rows((out,), self._combined_index(out.device, False))[0]
+        return self._reversed_rearrange_torch(out)
+
+    def _reversed_rearrange_torch(self, out: torch.Tensor) -> torch.Tensor:
         idx = self._indices(out.device, False)
         if self.text_length == 0:
             return out.index_select(-2, idx)
