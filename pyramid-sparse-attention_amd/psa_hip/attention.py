@@ -70,8 +70,13 @@ class PSAConfig:
 def draw_sample_offsets(B: int, H: int, block: int, keep: int, device, generator=None) -> torch.Tensor:
     """`keep` distinct in-block offsets per (b, h), int32 [B,H,keep]; every block of a head uses the
     same offsets.  reference: src/psa_triton/attention.py:132-133 (rand -> topk)."""
-    r = torch.rand(B, H, 1, block, device=device, generator=generator)
-    return torch.topk(r, keep, dim=3).indices.view(B, H, keep).to(torch.int32).contiguous()
+    if generator is not None and generator.device.type != "cpu":
+        r = torch.rand(B, H, 1, block, device=device, generator=generator)
+        return torch.topk(r, keep, dim=3).indices.view(B, H, keep).to(torch.int32).contiguous()
+    # Drawn on the host (default or given CPU generator): B*H*block numbers.  On the device the rand -> topk ->
+    # convert chain costs five launches and ~55 us per call, twice per layer, next to a 1 ms layer.
+    r = torch.rand(B, H, block, generator=generator)
+    return torch.topk(r, keep, dim=2).indices.to(torch.int32).contiguous().to(device, non_blocking=True)
 
 
 def _compute_attention_pooling(q, k, v, config, sample_offsets=None):
