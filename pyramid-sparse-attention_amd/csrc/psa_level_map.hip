@@ -35,11 +35,61 @@ __device__ __forceinline__ uint32_t desc_key(float s) {
   return ~u;                                   // descending
 }
 
+// Stable descending order of one row of scores: sw[i] / sidx[i] = score and column of sorted position i.
+// The 64-bit keys (inverted score bits, column) are unique, so every correct sort gives the same order.
+// Rows of up to 256 scores are ranked by counting (one pass of N comparisons per score, no barriers inside);
+// longer rows (32-key blocks: 1024 scores) are sorted in place by a bitonic network over key[0 .. Npad), Npad the
+// next power of two, padded with keys that sort last: N/2 compare-exchanges per stage instead of N comparisons
+// per score (1024 scores: 55 stages of 2 exchanges per thread against 4096 comparisons per thread).
+constexpr int RANK_SORT_MAX = 256;
+__host__ __device__ inline int sort_pad(int N) {
+  if (N <= RANK_SORT_MAX) return N;
+  int n = 1;
+  while (n < N) n <<= 1;
+  return n;
+}
+__device__ __forceinline__ void sort_row_desc(uint64_t* key, float* sw, int* sidx, const float* src, int N, int tid, int nt) {
+  const int Npad = sort_pad(N);
+  for (int j = tid; j < Npad; j += nt) key[j] = j < N ? (((uint64_t)desc_key(src[j]) << 32) | (uint32_t)j) : ~0ull;
+  __syncthreads();
+  if (N <= RANK_SORT_MAX) {
+    for (int j = tid; j < N; j += nt) {
+      const uint64_t kj = key[j];
+      int rank = 0;
+      for (int i = 0; i < N; ++i) rank += key[i] < kj ? 1 : 0;
+      sw[rank] = src[j];
+      sidx[rank] = j;
+    }
+  } else {
+    for (int k = 2; k <= Npad; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        for (int e = tid; e < (Npad >> 1); e += nt) {
+          // pair e of this stage: i has bit j clear, its partner is i + j; ascending where bit k of i is clear
+          const int i = ((e & ~(j - 1)) << 1) | (e & (j - 1));
+          const uint64_t a = key[i], b = key[i + j];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) {
+            key[i] = b;
+            key[i + j] = a;
+          }
+        }
+        __syncthreads();
+      }
+    }
+    for (int i = tid; i < N; i += nt) {
+      const int col = (int)(uint32_t)key[i];
+      sidx[i] = col;
+      sw[i] = src[col];
+    }
+  }
+  __syncthreads();
+}
+
 __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int N = p.Nk;
-  uint64_t* key = (uint64_t*)smem;            // [N]
-  float* sw = (float*)(key + N);              // [N] scores in sorted order
+  uint64_t* key = (uint64_t*)smem;            // [sort_pad(N)]
+  float* sw = (float*)(key + sort_pad(N));    // [N] scores in sorted order
   int* sidx = (int*)(sw + N);                 // [N] column of sorted position
   float* c32 = (float*)(sidx + N);            // [N] prefix sums
   __shared__ int s_cnt[PSA_MAX_LEVEL_ITEMS];
@@ -50,16 +100,7 @@ __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
   const float* src = p.scores + row * N;
 
   if (tid < PSA_MAX_LEVEL_ITEMS) s_cnt[tid] = 0;
-  for (int j = tid; j < N; j += nt) key[j] = ((uint64_t)desc_key(src[j]) << 32) | (uint32_t)j;
-  __syncthreads();
-  for (int j = tid; j < N; j += nt) {
-    const uint64_t kj = key[j];
-    int rank = 0;
-    for (int i = 0; i < N; ++i) rank += key[i] < kj ? 1 : 0;
-    sw[rank] = src[j];
-    sidx[rank] = j;
-  }
-  __syncthreads();
+  sort_row_desc(key, sw, sidx, src, N, tid, nt);
 
   if (p.mode == PSA_MODE_THRESHOLDBOUND) {
     if (tid == 0) {
@@ -208,7 +249,7 @@ extern "C" int psa_level_map(const float* scores, void* map_out, int map_elem_by
       }
     }
   }
-  size_t shmem = (size_t)Nk * (8 + 4 + 4 + 4);
+  size_t shmem = (size_t)sort_pad(Nk) * 8 + (size_t)Nk * (4 + 4 + 4);
   if (shmem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map: cannot reserve %zu bytes of LDS", shmem);
@@ -239,23 +280,14 @@ __global__ __launch_bounds__(256) void psa_level_map_qwen_kernel(QwenMapParams p
   extern __shared__ __align__(16) unsigned char smem[];
   const int N = p.S;
   uint64_t* key = (uint64_t*)smem;
-  float* sw = (float*)(key + N);
+  float* sw = (float*)(key + sort_pad(N));
   int* sidx = (int*)(sw + N);
   float* c32 = (float*)(sidx + N);
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t row = blockIdx.x;
   const int i_row = (int)(row % N);
   const float* src = p.scores + row * N;
-  for (int j = tid; j < N; j += nt) key[j] = ((uint64_t)desc_key(src[j]) << 32) | (uint32_t)j;
-  __syncthreads();
-  for (int j = tid; j < N; j += nt) {
-    const uint64_t kj = key[j];
-    int rank = 0;
-    for (int i = 0; i < N; ++i) rank += key[i] < kj ? 1 : 0;
-    sw[rank] = src[j];
-    sidx[rank] = j;
-  }
-  __syncthreads();
+  sort_row_desc(key, sw, sidx, src, N, tid, nt);
   if (p.mode == PSA_MODE_THRESHOLDBOUND) {
     if (tid == 0) {
       double acc = 0.0;
@@ -319,7 +351,7 @@ extern "C" int psa_level_map_qwen(const float* scores, void* map_out, int map_el
     }
     p.hi[t] = (float)item_hi[t];
   }
-  size_t shmem = (size_t)S * 20;
+  size_t shmem = (size_t)sort_pad(S) * 8 + (size_t)S * 12;
   if (shmem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_qwen_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map_qwen: cannot reserve %zu bytes of LDS", shmem);
