@@ -94,6 +94,7 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
     const int e = (slot0 + n) & (keep_n - 1);
     my_off[n] = ok ? ok[e] : e;
   }
+  const int last_off = ok ? ok[keep_n - 1] : keep_n - 1;
   auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
     const int r0 = t * TK + slot0;
     const bool inside = (t + 1) * TK <= Ns && ((((t + 1) * TK - 1) >> kn_log2) + 1) * bn <= Lk;  // uniform
@@ -102,13 +103,10 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
     for (int n = 0; n < RPL; ++n) {
       int src = grp_row + my_off[n];
       if (!inside) {
-        // padding keys replicate the last sampled key; rows past the sequence end clamp to its last row
-        int r = r0 + n;
-        if (r >= Ns) {
-          r = Ns - 1;
-          const int e = r & (keep_n - 1);
-          src = (r >> kn_log2) * bn + (ok ? ok[e] : e);
-        }
+        // padding keys replicate the last sampled key (Ns is a multiple of keep_n, so that is entry keep_n - 1 of
+        // the offset table: looked up once, before the loop - a global load in here would make the compiler wait
+        // for every copy in flight before each copy); rows past the sequence end clamp to its last row
+        if (r0 + n >= Ns) src = ((Ns - 1) >> kn_log2) * bn + last_off;
         src = src < Lk ? src : Lk - 1;
       }
       psa_tiles::lds_copy16(kb, (uint32_t)src * kstrb + f_chunk, psa_tiles::lds_addr_of(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR));
