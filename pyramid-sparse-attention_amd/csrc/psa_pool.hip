@@ -73,10 +73,12 @@ __global__ __launch_bounds__(256) void psa_pool_kernel(PoolParams p) {
   bf16_t* d4 = d2 + BH * (p.npad >> 1) * D;
   bf16_t* d8 = d4 + BH * (p.npad >> 2) * D;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) *(u32x4*)(d2 + ((int64_t)bh * (p.npad >> 1) + g * 4 + i) * D + c * 8) = o2[i];
+  // streaming stores: the pooled rows are not read again by this kernel and would only push the inputs of the
+  // next rows out of the caches (measured at the Wan2.1 shape: 70 -> 55 us)
+  for (int i = 0; i < 4; ++i) __builtin_nontemporal_store(o2[i], (u32x4*)(d2 + ((int64_t)bh * (p.npad >> 1) + g * 4 + i) * D + c * 8));
 #pragma unroll
-  for (int i = 0; i < 2; ++i) *(u32x4*)(d4 + ((int64_t)bh * (p.npad >> 2) + g * 2 + i) * D + c * 8) = o4[i];
-  *(u32x4*)(d8 + ((int64_t)bh * (p.npad >> 3) + g) * D + c * 8) = o8;
+  for (int i = 0; i < 2; ++i) __builtin_nontemporal_store(o4[i], (u32x4*)(d4 + ((int64_t)bh * (p.npad >> 2) + g * 2 + i) * D + c * 8));
+  __builtin_nontemporal_store(o8, (u32x4*)(d8 + ((int64_t)bh * (p.npad >> 3) + g) * D + c * 8));
 }
 
 extern "C" int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_pool, int B, int Hkv, int L, int D,

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void psa_gather_rows_kernel(GatherParams p) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int i = i0 + u * rows_per_wg + r;
-      if (i < p.L) *(u32x4*)(dst + (int64_t)i * p.d_sl[z]) = w[u];
+      if (i < p.L) __builtin_nontemporal_store(w[u], (u32x4*)(dst + (int64_t)i * p.d_sl[z]));  // streaming: written once, read by later kernels
     }
   }
 }
