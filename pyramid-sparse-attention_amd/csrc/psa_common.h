@@ -75,6 +75,12 @@ __device__ __forceinline__ float half_wave_max(float v) {
   half_wave_swap(v, lo, hi);
   return fmaxf(lo, hi);
 }
+// Maxima over both half-waves of a and of b with one exchange: lanes 0-31 return it for a, lanes 32-63 for b.
+__device__ __forceinline__ float half_wave_max_pair(float a, float b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+  const uint32_t r0 = r[0], r1 = r[1];  // r0 = (a low half, b low half), r1 = (a high half, b high half)
+  return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
 __device__ __forceinline__ float half_wave_sum(float v) {
   float lo, hi;
   half_wave_swap(v, lo, hi);

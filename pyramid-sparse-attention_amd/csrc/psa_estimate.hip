@@ -11,8 +11,8 @@
 // double-buffered LDS (one barrier per tile).  The key range is cut into 1, 2 or 4 shares (grid z) so that
 // the launch fills the chip; the row maxima of the shares are combined by kernel 2.  As in the forward
 // kernel the transposed product S^T = K Q^T is computed, so a lane holds 16 keys of one query row and a
-// key-group maximum is an in-lane v_max3 chain plus one half-wave exchange.  The group maxima go to an
-// fp32 workspace laid out [key group][query row] (128-byte coalesced stores, issued one tile late).
+// key-group maximum is an in-lane v_max3 chain plus a half-wave exchange shared by two key groups.  The group
+// maxima go to an fp32 workspace laid out [key group][query row] (coalesced stores, issued one tile late).
 // Kernel 2 (HBM-bound, reads the workspace once): per (query group, key group) the maximum over the
 // group's rows of R - m, exp2, row sum in a fixed order, normalisation.
 #include "psa_common.h"
@@ -50,13 +50,45 @@ __device__ __forceinline__ int sampled_src(int r, int n_real, int keep_log2, int
 // copied from global memory straight into LDS, double buffered, in the padded + swizzled tile layout of
 // psa_tiles.h (shared with the attention kernels): the 128-bit operand reads are bank-conflict free and their
 // addresses are lane base + immediate.
+//
+// Three waves share a SIMD, and whatever a wave executes outside its MFMA stream (copy addresses, the group
+// maxima, store addresses) advances slowly while the other two stream MFMAs: that part is kept to a few dozen
+// vector instructions per tile.  The copy and store addresses are a per-tile scalar base plus a lane offset
+// computed once; the two 32-key chunks of a tile are multiplied one after the other, so that the maxima of
+// the first chunk are taken in the shadow of the second chunk's MFMAs; and one half-wave exchange serves two
+// key groups (lanes 0-31 keep the maximum of the even group, lanes 32-63 that of the odd one).
 constexpr int E_STAGES = 2;
 
-template <int D>
+// piece k (0..7) of the in-lane maxima of one 32-key chunk: NV = 1 << GPC values, 8 instructions in all.
+// Register i of the chunk holds key (i / 4) * 8 + 4 * (lane / 32) + i % 4, so the keys of an 8-key octet are
+// registers 4o..4o+3 of both half-waves.
+template <int GPC>
+__device__ __forceinline__ void chunk_max_piece(const f32x16& sc, float (&val)[1 << GPC], float (&tmp)[3], int k) {
+  if constexpr (GPC == 0) {
+    if (k == 0) val[0] = max3f(sc[0], sc[1], sc[2]);
+    else if (k < 7) val[0] = max3f(val[0], sc[2 * k + 1], sc[2 * k + 2]);
+    else val[0] = fmaxf(val[0], sc[15]);
+  } else if constexpr (GPC == 1) {
+    const int o = k >> 2, j = k & 3;
+    if (j == 0) tmp[0] = max3f(sc[8 * o], sc[8 * o + 1], sc[8 * o + 2]);
+    else if (j == 1) tmp[1] = max3f(sc[8 * o + 3], sc[8 * o + 4], sc[8 * o + 5]);
+    else if (j == 2) tmp[2] = fmaxf(sc[8 * o + 6], sc[8 * o + 7]);
+    else val[o] = max3f(tmp[0], tmp[1], tmp[2]);
+  } else {
+    const int o = k >> 1;
+    if ((k & 1) == 0) tmp[0] = max3f(sc[4 * o], sc[4 * o + 1], sc[4 * o + 2]);
+    else val[o] = fmaxf(tmp[0], sc[4 * o + 3]);
+  }
+}
+
+template <int D, int GPC>
 __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
   using G = psa_tiles::LtGeom<D>;
   constexpr int KK = D / 16, RS = 2;  // RS sets of 32 query rows per wave
   constexpr int E_TILE = G::TILE, E_ISTR = psa_tiles::LT_ISTR, RPL = G::RPL;
+  constexpr int NV = 1 << GPC;        // key groups per 32-key chunk = registers of group maxima per row set and tile
+  constexpr int PPS = 8 / KK;         // pieces of the first chunk's maxima per k-step of the second chunk
+  static_assert(8 % KK == 0 && PPS >= 1, "the maxima of a chunk are 8 pieces");
   __shared__ __align__(16) unsigned char smem[E_STAGES * E_TILE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -64,7 +96,8 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
   const int bh = blockIdx.y;
   const int h = bh % p.Hq, b = bh / p.Hq;
   const int hk = h / (p.Hq / p.Hkv);
-  const int keep_m = 1 << p.keep_m_log2, keep_n = 1 << p.keep_n_log2;
+  const int keep_m = 1 << p.keep_m_log2;
+  constexpr int kn_log2 = 5 - GPC, keep_n = 1 << kn_log2;
 
   // Q fragments: lane holds Q[row l32 of set rs][16*kk + 8*hh .. +8]
   const int row0 = blockIdx.x * (4 * 32 * RS) + wave * (32 * RS);
@@ -83,33 +116,43 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
   const char* kb = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
   const uint32_t kstrb = (uint32_t)p.k_sl * 2u;
   const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * keep_n : nullptr;
-  const int Ns = p.Ns, Lk = p.Lk, bn = p.bn, kn_log2 = p.keep_n_log2;
+  const int Ns = p.Ns, Lk = p.Lk, bn = p.bn;
 
-  // fetch: wave w copies the 16-row group w of a tile, one block per instruction
+  // fetch: wave w copies the 16-row group w of a tile, one block per instruction.  A tile of 64 sampled keys
+  // spans 64 / keep_n whole key groups, so the source row of a tile slot is t * (64 / keep_n) * block_n plus a
+  // per-lane constant: the copies of a tile inside the sequence cost no vector arithmetic.
   const uint32_t f_chunk = psa_tiles::lt_fetch_chunk<D>(lane);
   const int slot0 = wave * 16 + psa_tiles::lt_fetch_row<D>(lane);  // first of this lane's consecutive tile slots
   int my_off[RPL];
+  uint32_t c_off[RPL];
 #pragma unroll
   for (int n = 0; n < RPL; ++n) {
     const int e = (slot0 + n) & (keep_n - 1);
     my_off[n] = ok ? ok[e] : e;
+    c_off[n] = (uint32_t)((slot0 >> kn_log2) * bn + my_off[n]) * kstrb + f_chunk;
   }
   const int last_off = ok ? ok[keep_n - 1] : keep_n - 1;
+  const uint64_t tile_step = (uint64_t)((TK >> kn_log2) * bn) * kstrb;  // bytes between the key groups of consecutive tiles
   auto issue_tile = [&](int t, int stage) __attribute__((always_inline)) {
-    const int r0 = t * TK + slot0;
     const bool inside = (t + 1) * TK <= Ns && ((((t + 1) * TK - 1) >> kn_log2) + 1) * bn <= Lk;  // uniform
-    const int grp_row = (r0 >> kn_log2) * bn;
+    if (inside) {
+      const char* tb = kb + (uint64_t)t * tile_step;
 #pragma unroll
-    for (int n = 0; n < RPL; ++n) {
-      int src = grp_row + my_off[n];
-      if (!inside) {
-        // padding keys replicate the last sampled key (Ns is a multiple of keep_n, so that is entry keep_n - 1 of
-        // the offset table: looked up once, before the loop - a global load in here would make the compiler wait
-        // for every copy in flight before each copy); rows past the sequence end clamp to its last row
+      for (int n = 0; n < RPL; ++n)
+        psa_tiles::lds_copy16(tb, c_off[n], psa_tiles::lds_addr_of(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR));
+    } else {
+      // padding keys replicate the last sampled key (Ns is a multiple of keep_n, so that is entry keep_n - 1 of
+      // the offset table: looked up once, before the loop - a global load in here would make the compiler wait
+      // for every copy in flight before each copy); rows past the sequence end clamp to its last row
+      const int r0 = t * TK + slot0;
+      const int grp_row = (r0 >> kn_log2) * bn;
+#pragma unroll
+      for (int n = 0; n < RPL; ++n) {
+        int src = grp_row + my_off[n];
         if (r0 + n >= Ns) src = ((Ns - 1) >> kn_log2) * bn + last_off;
         src = src < Lk ? src : Lk - 1;
+        psa_tiles::lds_copy16(kb, (uint32_t)src * kstrb + f_chunk, psa_tiles::lds_addr_of(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR));
       }
-      psa_tiles::lds_copy16(kb, (uint32_t)src * kstrb + f_chunk, psa_tiles::lds_addr_of(smem + stage * E_TILE + (wave * RPL + n) * E_ISTR));
     }
   };
   // K operand of k-step kk for tile slots l32 and l32 + 32: k_off[kk & 1] + 64 * (kk >> 1) (+ G::HALF)
@@ -117,34 +160,24 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
   psa_tiles::lt_row_operand<D>(l32, hh, k_off);
 
   const int T = p.Ns_pad / TK;
-  const int gpc_log2 = 5 - p.keep_n_log2;  // key groups per 32-key chunk (1, 2 or 4)
-  float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + row0 + l32;
+  // workspace rows of this wave: uniform base + lane offset (lanes 32-63 store for the odd key group of a pair)
   const int64_t rts = p.Ms_pad;
+  float* const rt_u = p.rt + (int64_t)bh * p.n_d * rts + row0;
+  const uint32_t st_off = (uint32_t)hh * (uint32_t)rts + (uint32_t)l32;
   float m_run[RS];
 #pragma unroll
   for (int rs = 0; rs < RS; ++rs) m_run[rs] = -INFINITY;
   const float qk_scale = p.qk_scale;
 
   // group maxima of the previous tile, written one tile late so that the stores' latency hides behind the MFMAs:
-  // per (row set, 32-key chunk) a lane owns at most 2 values (it stores for key group jbase + 2*i + hh, or for
-  // jbase when there is one group per chunk)
-  float pend[RS][2][2];
+  // register pr of a row set holds key groups 2 * pr (lanes 0-31) and 2 * pr + 1 (lanes 32-63) of the tile
+  float pend[RS][NV];
   auto flush = [&](int tp) __attribute__((always_inline)) {
+    float* const tb = rt_u + (int64_t)tp * (2 * NV) * rts;
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs)
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const int jbase = (tp * 2 + c) << gpc_log2;
-        float* rto = rt + rs * 32;
-        if (gpc_log2 == 0) {
-          if (hh == 0) rto[(int64_t)jbase * rts] = pend[rs][c][0];
-        } else if (gpc_log2 == 1) {
-          rto[(int64_t)(jbase + hh) * rts] = pend[rs][c][0];
-        } else {
-          rto[(int64_t)(jbase + hh) * rts] = pend[rs][c][0];
-          rto[(int64_t)(jbase + 2 + hh) * rts] = pend[rs][c][1];
-        }
-      }
+      for (int pr = 0; pr < NV; ++pr) (tb + (int64_t)(2 * pr) * rts + rs * 32)[st_off] = pend[rs][pr];
   };
 
   // this workgroup's share of the key tiles
@@ -153,73 +186,60 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
   issue_tile(t_begin, t_begin & 1);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int t = t_begin; t < t_end; ++t) {
     // invariant: stage t&1 holds tile t and every wave is done with the other stage
     if (t + 1 < t_end) issue_tile(t + 1, (t + 1) & 1);
     if (t > t_begin) flush(t - 1);
 
     PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem) + (t & 1) * E_TILE;
+    // step i = chunk c * KK + k-step kk; its operand is requested two steps (four MFMAs) ahead
+    auto kread = [&](int i) __attribute__((always_inline)) {
+      const int c = i / KK, kk = i % KK;
+      return *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
+    };
     f32x16 s[RS][2];
+    float val[RS][2][NV], tmp[RS][3];
+    bf16x8 ka[3];
+    ka[0] = kread(0);
+    ka[1] = kread(1);
 #pragma unroll
-    for (int rs = 0; rs < RS; ++rs)
+    for (int i = 0; i < 2 * KK; ++i) {
+      const int c = i / KK, kk = i % KK;
+      if (i + 2 < 2 * KK) ka[(i + 2) % 3] = kread(i + 2);
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+      for (int rs = 0; rs < RS; ++rs) s[rs][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[i % 3], qf[rs][kk], kk == 0 ? zero16 : s[rs][c], 0, 0, 0);
+      if (c == 1) {
+        __builtin_amdgcn_sched_barrier(0);  // after this step's MFMAs: the first piece waits for chunk 0's last results
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[rs][c][i] = 0.f;
-    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + G::HALF);
+        for (int k = kk * PPS; k < (kk + 1) * PPS; ++k)
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      bf16x8 n0 = a0, n1 = a1;
-      if (kk + 1 < KK) {
-        n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
-        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + G::HALF);
+          for (int rs = 0; rs < RS; ++rs) chunk_max_piece<GPC>(s[rs][0], val[rs][0], tmp[rs], k);
       }
-#pragma unroll
-      for (int rs = 0; rs < RS; ++rs) {
-        s[rs][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[rs][kk], s[rs][0], 0, 0, 0);
-        s[rs][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[rs][kk], s[rs][1], 0, 0, 0);
-      }
-      a0 = n0;
-      a1 = n1;
+      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
+    for (int k = 0; k < 8; ++k)
+#pragma unroll
+      for (int rs = 0; rs < RS; ++rs) chunk_max_piece<GPC>(s[rs][1], val[rs][1], tmp[rs], k);
+#pragma unroll
     for (int rs = 0; rs < RS; ++rs)
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        // register i holds key (i/4)*8 + hh*4 + i%4 of this chunk: 8-key octets are registers 4o..4o+3
-        const f32x16& sc = s[rs][c];
-        if (gpc_log2 == 0) {
-          float v = sc[0];
-#pragma unroll
-          for (int i = 1; i < 15; i += 2) v = max3f(v, sc[i], sc[i + 1]);
-          v = half_wave_max(fmaxf(v, sc[15])) * qk_scale;
-          m_run[rs] = fmaxf(m_run[rs], v);
-          pend[rs][c][0] = v;
-        } else if (gpc_log2 == 1) {
-          float v0 = max3f(max3f(sc[0], sc[1], sc[2]), max3f(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
-          float v1 = max3f(max3f(sc[8], sc[9], sc[10]), max3f(sc[11], sc[12], sc[13]), fmaxf(sc[14], sc[15]));
-          v0 = half_wave_max(v0) * qk_scale;
-          v1 = half_wave_max(v1) * qk_scale;
-          m_run[rs] = max3f(m_run[rs], v0, v1);
-          pend[rs][c][0] = hh ? v1 : v0;
-        } else {
-          float v[4];
-#pragma unroll
-          for (int o = 0; o < 4; ++o) {
-            v[o] = half_wave_max(fmaxf(max3f(sc[4 * o], sc[4 * o + 1], sc[4 * o + 2]), sc[4 * o + 3])) * qk_scale;
-            m_run[rs] = fmaxf(m_run[rs], v[o]);
-          }
-          pend[rs][c][0] = hh ? v[1] : v[0];
-          pend[rs][c][1] = hh ? v[3] : v[2];
-        }
+      for (int pr = 0; pr < NV; ++pr) {
+        // the tile's 2 * NV key groups in order: chunk 0's, then chunk 1's
+        const int e0 = 2 * pr, e1 = 2 * pr + 1;
+        const float v = half_wave_max_pair(val[rs][e0 / NV][e0 % NV], val[rs][e1 / NV][e1 % NV]) * qk_scale;
+        m_run[rs] = fmaxf(m_run[rs], v);
+        pend[rs][pr] = v;
       }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // the copies of tile t+1 (and the stores of tile t-1) were issued a tile ago
     __syncthreads();
   }
   if (t_end > t_begin) flush(t_end - 1);
-  if (hh == 0) {
 #pragma unroll
-    for (int rs = 0; rs < RS; ++rs) p.mrow[((int64_t)bh * p.ksplit + ks) * p.Ms_pad + row0 + rs * 32 + l32] = m_run[rs];
+  for (int rs = 0; rs < RS; ++rs) {
+    const float m = half_wave_max(m_run[rs]);  // the halves saw different key groups
+    if (hh == 0) p.mrow[((int64_t)bh * p.ksplit + ks) * p.Ms_pad + row0 + rs * 32 + l32] = m;
   }
 }
 
@@ -277,7 +297,11 @@ int launch_est(EstParams& p, int B, hipStream_t stream) {
   const int tiles = p.Ns_pad / TK;
   while (p.ksplit < EST_MAX_KSPLIT && wgs * p.ksplit < 3 * 256 && tiles / (p.ksplit * 2) >= 8) p.ksplit *= 2;
   grid.z = (unsigned)p.ksplit;
-  hipLaunchKernelGGL(psa_est_gemm_lds_kernel<D>, grid, dim3(256), 0, stream, p);
+  switch (p.keep_n_log2) {
+    case 5: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 0>), grid, dim3(256), 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 1>), grid, dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 2>), grid, dim3(256), 0, stream, p); break;
+  }
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
   hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
