@@ -468,19 +468,20 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
   const float scale_log2 = p.scale_log2;
   const float bias = (float)lv;
-  const int spb = bm / 64;           // steps per q-block
-  const int n_steps = key_valid > 0 ? nq * spb : 0;
+  const int spb_log2 = bm >> 7;      // steps of 64 query rows per q-block: 1 (block_m 64) or 2 (128)
+  const int n_steps = key_valid > 0 ? nq << spb_log2 : 0;
   const uint32_t q_strb = (uint32_t)p.q_sl * 2u, do_strb = (uint32_t)p.do_sl * 2u;
 
   // step i -> (head, q-block, first query row)
   auto step_of = [&](int i, int& h, int& I, int& q0) __attribute__((always_inline)) {
-    const uint32_t ent = qlist[i / spb];
+    const uint32_t ent = qlist[i >> spb_log2];
     h = hk * n_rep + (int)(ent >> 16);
     I = (int)(ent & 0xffff);
-    q0 = I * bm + (i % spb) * 64;
+    q0 = I * bm + (i & ((1 << spb_log2) - 1)) * 64;
   };
   // rows of step i -> stage; the per-row lse / delta values come back in registers and are put into LDS later
   float lse_next = 0.f, del_next = 0.f;
+
   auto issue_step = [&](int i, int stage) __attribute__((always_inline)) {
     int h, I, q0;
     step_of(i, h, I, q0);
@@ -734,6 +735,8 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
                 PSA_ERR_UNSUPPORTED, "psa_bwd: tensors must be 16-byte aligned with strides that are multiples of 8 elements");
   PSA_REQUIRE((int64_t)L * k.stride_l * 2 < (1ll << 32) && (int64_t)L * v.stride_l * 2 < (1ll << 32), PSA_ERR_UNSUPPORTED,
               "psa_bwd: one (batch, head) slice of K/V must span less than 4 GiB");
+  PSA_REQUIRE((int64_t)L * q.stride_l * 2 < (1ll << 32) && (int64_t)L * dout.stride_l * 2 < (1ll << 32), PSA_ERR_UNSUPPORTED,
+              "psa_bwd: one (batch, head) slice of q / dout must span less than 4 GiB");
   const int Mq = (L + block_m - 1) / block_m, Nk = (L + block_n - 1) / block_n;
   PSA_REQUIRE(Nk <= 65535 && Mq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: more than 65535 blocks");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: B*Hq too large");

@@ -924,7 +924,9 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
   p.grp_bytes = 0;
   // two rows per workgroup when the head dim / block size have that kernel and both schedules fit into LDS
-  const bool two_group = D == 128 && block_m == 128 && total > 1 && pp_lds_bytes<128>(p.max_tiles, Nk) <= 160 * 1024 && !PSA_FWD_ONE_GROUP;
+  // (that kernel forms its copy offsets with 24-bit multiplies: row index and row stride in bytes must fit)
+  const bool two_group = D == 128 && block_m == 128 && total > 1 && pp_lds_bytes<128>(p.max_tiles, Nk) <= 160 * 1024 && !PSA_FWD_ONE_GROUP &&
+                         (int64_t)Nk * block_n < (1 << 24) && k.stride_l * 2 < (1 << 24) && v.stride_l * 2 < (1 << 24);
   if (two_group) p.wg_chunk = (p.wg_chunk + 1) & ~1;  // pairs never straddle two groups of rows
   p.order = nullptr;
   if (workspace != nullptr && map != nullptr && total > 8 * 32) {
