@@ -48,12 +48,14 @@ __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem,
   const int share = ((jmax + 64 * NW - 1) / (64 * NW)) * 64;
   const int j_lo = wave * share, j_hi = (wave + 1) * share < jmax ? (wave + 1) * share : jmax;
   int cnt[4] = {0, 0, 0, 0};
+  int lvl_first = 0;  // the first 64 entries of the share stay in a register for the second pass
   if (map == nullptr) {
     cnt[0] = j_hi > j_lo ? j_hi - j_lo : 0;
   } else {
     for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
       const int j = j0 + lane;
       const int lvl = j < j_hi ? load_map(map, mrow + j, map_elem) : 0;
+      if (j0 == j_lo) lvl_first = lvl;
 #pragma unroll
       for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
     }
@@ -87,7 +89,8 @@ __device__ __forceinline__ int build_row_schedule(const void* map, int map_elem,
       const uint64_t lt_mask = (1ull << lane) - 1ull;
       for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
         const int j = j0 + lane;
-        const int lvl = j < j_hi ? load_map(map, mrow + j, map_elem) : 0;
+        int lvl = lvl_first;
+        if (j0 != j_lo) lvl = j < j_hi ? load_map(map, mrow + j, map_elem) : 0;
 #pragma unroll
         for (int lv = 0; lv < 4; ++lv) {
           const uint64_t bal = __ballot(lvl == (1 << lv));
