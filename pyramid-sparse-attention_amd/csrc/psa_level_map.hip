@@ -85,6 +85,39 @@ __device__ __forceinline__ void sort_row_desc(uint64_t* key, float* sw, int* sid
   __syncthreads();
 }
 
+// Prefix sums of the sorted scores, accumulated strictly sequentially in fp64 and rounded to fp32 (the order
+// matters for bit-exactness).  All threads widen the scores into `wide` (the sort's key buffer, free by now) and
+// round the sums afterwards, so that the dependent chain one lane has to run is a load, an addition and a store
+// per two scores; that lane runs it at raised wave priority, because up to seven other waves compete with it for
+// every instruction slot of the SIMD and the rest of its workgroup waits for it.
+__device__ __forceinline__ void row_prefix_sums(double* wide, const float* sw, float* c32, int N, int tid, int nt) {
+  typedef double f64x2 __attribute__((ext_vector_type(2)));
+  for (int i = tid; i < N; i += nt) wide[i] = (double)sw[i];
+  __syncthreads();
+  if (tid == 0) {
+    __builtin_amdgcn_s_setprio(3);
+    double acc = 0.0;
+    int i = 0;
+    for (; i + 4 <= N; i += 4) {
+      const f64x2 w0 = *(const f64x2*)(wide + i), w1 = *(const f64x2*)(wide + i + 2);
+      const double a0 = acc + w0[0];
+      const double a1 = a0 + w0[1];
+      const double a2 = a1 + w1[0];
+      acc = a2 + w1[1];
+      *(f64x2*)(wide + i) = f64x2{a0, a1};
+      *(f64x2*)(wide + i + 2) = f64x2{a2, acc};
+    }
+    for (; i < N; ++i) {
+      acc += wide[i];
+      wide[i] = acc;
+    }
+    __builtin_amdgcn_s_setprio(0);
+  }
+  __syncthreads();
+  for (int i = tid; i < N; i += nt) c32[i] = (float)wide[i];
+  __syncthreads();
+}
+
 __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int N = p.Nk;
@@ -103,40 +136,30 @@ __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
   sort_row_desc(key, sw, sidx, src, N, tid, nt);
 
   if (p.mode == PSA_MODE_THRESHOLDBOUND) {
-    if (tid == 0) {
-      // strictly sequential fp64 accumulation (the order matters for bit-exactness); the LDS traffic is
-      // batched four values at a time so that only the additions form the dependent chain
-      double acc = 0.0;
-      int i = 0;
-      for (; i + 4 <= N; i += 4) {
-        const float w0 = sw[i], w1 = sw[i + 1], w2 = sw[i + 2], w3 = sw[i + 3];
-        const double a0 = acc + (double)w0;
-        const double a1 = a0 + (double)w1;
-        const double a2 = a1 + (double)w2;
-        acc = a2 + (double)w3;
-        c32[i] = (float)a0; c32[i + 1] = (float)a1; c32[i + 2] = (float)a2; c32[i + 3] = (float)acc;
-      }
-      for (; i < N; ++i) {
-        acc += (double)sw[i];
-        c32[i] = (float)acc;
-      }
-    }
-    __syncthreads();
+    row_prefix_sums((double*)key, sw, c32, N, tid, nt);
     const float total = c32[N - 1];
+    // positions whose cumulative ratio is within each item's bound: one ballot per item and pass, one LDS
+    // atomic per wave and item (integer counts: the order of the additions does not matter)
     int local[PSA_MAX_LEVEL_ITEMS];
 #pragma unroll
     for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t) local[t] = 0;
-    for (int i = tid; i < N; i += nt) {
-      const float r = c32[i] / total;
+    for (int i0 = 0; i0 < N; i0 += nt) {
+      const int i = i0 + tid;
+      const float r = i < N ? c32[i] / total : 0.f;
 #pragma unroll
       for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t)
-        if (t < p.n_items && r <= p.thr[t]) local[t]++;
+        if (t < p.n_items) local[t] += __popcll(__ballot(i < N && r <= p.thr[t]));
     }
+    if ((tid & 63) == 0) {
 #pragma unroll
-    for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t)
-      if (t < p.n_items && local[t]) atomicAdd(&s_cnt[t], local[t]);
+      for (int t = 0; t < PSA_MAX_LEVEL_ITEMS; ++t)
+        if (t < p.n_items && local[t]) atomicAdd(&s_cnt[t], local[t]);
+    }
     __syncthreads();
     if (tid == 0) {
+      // a short dependent chain in one lane while the workgroup waits: raised priority, and no integer
+      // division for the usual power-of-two alignments
+      __builtin_amdgcn_s_setprio(3);
       int last = 0;
       for (int t = 0; t < p.n_items; ++t) {
         const int cnt = s_cnt[t];
@@ -147,11 +170,12 @@ __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
         if (al > 1) {
           int len = end0 - start;
           len = len > 0 ? len : 0;
-          const int rem = len % al;
+          const bool pow2 = (al & (al - 1)) == 0;
+          const int rem = pow2 ? (len & (al - 1)) : len % al;
           if (rem) len += al - rem;
           end = start + len;
           end = end < N ? end : N;
-          if (end == N) end = start + ((end - start) / al) * al;
+          if (end == N) end = start + (pow2 ? ((end - start) & ~(al - 1)) : ((end - start) / al) * al);
         } else {
           end = end0 < 0 ? 0 : (end0 > N ? N : end0);
           end = end > start ? end : start;
@@ -161,6 +185,7 @@ __global__ __launch_bounds__(256) void psa_level_map_kernel(LevelMapParams p) {
         s_iv[t][1] = end;
         last = end;
       }
+      __builtin_amdgcn_s_setprio(0);
     }
   } else {
     if (tid < p.n_items) {
@@ -289,14 +314,7 @@ __global__ __launch_bounds__(256) void psa_level_map_qwen_kernel(QwenMapParams p
   const float* src = p.scores + row * N;
   sort_row_desc(key, sw, sidx, src, N, tid, nt);
   if (p.mode == PSA_MODE_THRESHOLDBOUND) {
-    if (tid == 0) {
-      double acc = 0.0;
-      for (int i = 0; i < N; ++i) {
-        acc += (double)sw[i];
-        c32[i] = (float)acc;
-      }
-    }
-    __syncthreads();
+    row_prefix_sums((double*)key, sw, c32, N, tid, nt);
   }
   const float total = p.mode == PSA_MODE_THRESHOLDBOUND ? fmaxf(c32[N - 1], 1e-10f) : 1.f;
   const float valid_len = p.causal ? (float)(i_row + 1) : (float)N;
