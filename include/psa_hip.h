@@ -97,6 +97,19 @@ int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_
                   const double* item_hi, int align_div, int text_blocks, double min_full_attn_ratio,
                   psa_stream_t stream);
 
+/* psa_estimate_sampled followed by psa_level_map (dense map only) in two launches instead of three: the kernel that
+ * reduces the estimator's workspace to a row of scores goes on to rank that row while it is still in LDS.  The map
+ * [B, Hq, out_rows, out_cols] is the one psa_level_map computes from the scores psa_estimate_sampled returns, bit for
+ * bit; `scores` may be NULL when only the map is wanted.  Arguments as in the two functions (Nk = out_cols).
+ * Replaces the same reference code as they do (attn_with_pooling_optimized + transfer_attn_to_mask as called from
+ * reference src/psa_triton/attention.py:178-235). */
+int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k,
+                             float* scores, void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D,
+                             int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                             int out_rows, int out_cols, void* map_out, int map_elem_bytes, int mode, int n_items,
+                             const int32_t* item_level, const double* item_hi, int align_div, int text_blocks,
+                             double min_full_attn_ratio, psa_stream_t stream);
+
 /* Level map of the causal Qwen2.5-VL example: scores [bh, S, S] fp32 -> map [bh, S, S].  Items (level, lo, hi) in
  * dict order (host arrays).  PSA_MODE_TOPK: sorted positions [floor(len*lo), floor(len*hi)) get the level, len = row+1
  * if causal else S; PSA_MODE_THRESHOLDBOUND ("energybound"): positions whose cumulative ratio r satisfies

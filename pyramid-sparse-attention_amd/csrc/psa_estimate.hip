@@ -16,6 +16,7 @@
 // Kernel 2 (HBM-bound, reads the workspace once): per (query group, key group) the maximum over the
 // group's rows of R - m, exp2, row sum in a fixed order, normalisation.
 #include "psa_common.h"
+#include "psa_level_map_row.h"
 #include "psa_tiles.h"
 
 namespace {
@@ -247,10 +248,8 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
 // A lane reads 4 consecutive rows (16 bytes) of one key group, keep_m/4 neighbouring lanes cover the group's
 // rows (one contiguous run of the workspace), a wave 256/keep_m key groups per load; the maximum over the
 // group's rows is an in-lane maximum plus a butterfly over those lanes.
-__global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
-  extern __shared__ float s_e[];  // [n_d] un-normalised Po row
-  __shared__ float s_part[4];
-  const int i = blockIdx.x, bh = blockIdx.y;
+// Leaves the un-normalised row in s_e[0 .. n_d) and returns its sum (fixed summation order); 256 threads.
+__device__ __forceinline__ float est_reduce_row(const EstParams& p, float* s_e, float* s_part, int i, int bh) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lpg_log2 = p.keep_m_log2 - 2;            // lanes per key group
   const int quad = lane & ((1 << lpg_log2) - 1), sub = lane >> lpg_log2;
@@ -281,13 +280,41 @@ __global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
   for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
   if (lane == 0) s_part[wave] = part;
   __syncthreads();
-  const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+  return (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+}
+
+__global__ __launch_bounds__(256) void psa_est_reduce_kernel(EstParams p) {
+  extern __shared__ float s_e[];  // [n_d] un-normalised Po row
+  __shared__ float s_part[4];
+  const int i = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+  const float total = est_reduce_row(p, s_e, s_part, i, bh);
   float* dst = p.scores + ((int64_t)bh * p.out_rows + i) * p.out_cols;
   for (int j = tid; j < p.out_cols; j += 256) dst[j] = s_e[j] / total;
 }
 
+// The same, followed by the level map of the row while its scores are still in LDS: the workspace pass (HBM) of
+// one workgroup overlaps the sorting (VALU / LDS) of the others, and a launch and a round trip of the scores
+// through memory go away.  LDS: [level-map scratch: lm_bytes][n_d floats].  p.scores may be null.
+__global__ __launch_bounds__(256) void psa_est_reduce_map_kernel(EstParams p, LevelMapParams lp, int lm_bytes) {
+  extern __shared__ __align__(16) unsigned char smem_rm[];
+  __shared__ float s_part[4];
+  __shared__ int s_cnt[PSA_MAX_LEVEL_ITEMS];
+  __shared__ int s_iv[PSA_MAX_LEVEL_ITEMS][2];
+  float* s_e = (float*)(smem_rm + lm_bytes);
+  const int i = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+  const float total = est_reduce_row(p, s_e, s_part, i, bh);
+  const int64_t row = (int64_t)bh * p.out_rows + i;
+  for (int j = tid; j < p.out_cols; j += 256) {
+    const float v = s_e[j] / total;
+    s_e[j] = v;
+    if (p.scores) p.scores[row * p.out_cols + j] = v;
+  }
+  __syncthreads();
+  level_map_row(lp, s_e, row, smem_rm, s_cnt, s_iv, tid, 256);
+}
+
 template <int D>
-int launch_est(EstParams& p, int B, hipStream_t stream) {
+int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp) {
   const int rows_needed = p.out_rows << p.keep_m_log2;
   dim3 grid((unsigned)((rows_needed + 255) / 256), (unsigned)(B * p.Hq));
   // 256-row workgroups: cut the key range until about 3 workgroups per CU exist (the kernel's occupancy),
@@ -304,8 +331,19 @@ int launch_est(EstParams& p, int B, hipStream_t stream) {
   }
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
-  hipLaunchKernelGGL(psa_est_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * p.Hq)), dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
-  return psa_check_launch("psa_estimate_sampled (reduction)");
+  const dim3 rgrid((unsigned)p.out_rows, (unsigned)(B * p.Hq));
+  if (lp == nullptr) {
+    hipLaunchKernelGGL(psa_est_reduce_kernel, rgrid, dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
+    return psa_check_launch("psa_estimate_sampled (reduction)");
+  }
+  const size_t lm_bytes = (level_map_lds_bytes(lp->Nk) + 15) & ~(size_t)15;
+  const size_t shmem = lm_bytes + (size_t)p.n_d * sizeof(float);
+  if (shmem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)psa_est_reduce_map_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_estimate_sampled_map: cannot reserve %zu bytes of LDS", shmem);
+  }
+  hipLaunchKernelGGL(psa_est_reduce_map_kernel, rgrid, dim3(256), shmem, stream, p, *lp, (int)lm_bytes);
+  return psa_check_launch("psa_estimate_sampled_map (reduction + level map)");
 }
 
 struct EstGeom {
@@ -332,10 +370,11 @@ extern "C" int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, i
   return (int64_t)B * Hq * ((int64_t)g.n_d + EST_MAX_KSPLIT) * g.Ms_pad * (int64_t)sizeof(float);
 }
 
-extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
-                                    void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
-                                    int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
-  PSA_REQUIRE(q.ptr && k.ptr && scores && workspace, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
+namespace {
+int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores, void* workspace, int B, int Hq,
+            int Hkv, int Lq, int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale, int out_rows,
+            int out_cols, LevelMapParams* lp, psa_stream_t stream) {
+  PSA_REQUIRE(q.ptr && k.ptr && (scores || lp) && workspace, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Lq > 0 && Lk > 0, PSA_ERR_ARG, "psa_estimate_sampled: sizes must be positive");
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_estimate_sampled: Hq must be a multiple of Hkv");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: B*Hq too large");
@@ -363,5 +402,34 @@ extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t*
   p.qk_scale = sm_scale * 1.44269504f;
   p.rt = (float*)workspace;
   p.mrow = p.rt + (int64_t)B * Hq * g.n_d * g.Ms_pad;
-  return D == 128 ? launch_est<128>(p, B, (hipStream_t)stream) : launch_est<64>(p, B, (hipStream_t)stream);
+  if (lp != nullptr) {
+    PSA_REQUIRE(lp->Nk == out_cols, PSA_ERR_ARG, "psa_estimate_sampled_map: the map has %d columns, the scores %d", lp->Nk, out_cols);
+    lp->scores = nullptr;
+  }
+  return D == 128 ? launch_est<128>(p, B, (hipStream_t)stream, lp) : launch_est<64>(p, B, (hipStream_t)stream, lp);
+}
+}  // namespace
+
+extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
+                                    void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
+                                    int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
+  PSA_REQUIRE(scores, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
+  return est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale, out_rows,
+                 out_cols, nullptr, stream);
+}
+
+extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
+                                        void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
+                                        int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, void* map_out,
+                                        int map_elem_bytes, int mode, int n_items, const int32_t* item_level, const double* item_hi,
+                                        int align_div, int text_blocks, double min_full_attn_ratio, psa_stream_t stream) {
+  PSA_REQUIRE(map_out, PSA_ERR_ARG, "psa_estimate_sampled_map: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_estimate_sampled_map: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(out_cols > 0, PSA_ERR_ARG, "psa_estimate_sampled_map: out_cols must be positive");
+  LevelMapParams lp;
+  const int rc = level_map_fill_params(lp, out_cols, mode, n_items, item_level, item_hi, align_div, text_blocks, min_full_attn_ratio);
+  if (rc != PSA_OK) return rc;
+  lp.map_out = map_out; lp.map_elem = map_elem_bytes;
+  return est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale, out_rows,
+                 out_cols, &lp, stream);
 }

@@ -36,6 +36,12 @@ SIGNATURES = {
         [Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
          c_int, c_float, c_int, c_int, c_void_p],
     ),
+    "psa_estimate_sampled_map": (
+        c_int,
+        [Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int, c_int, c_double,
+         c_void_p],
+    ),
     "psa_level_map": (
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int,

@@ -104,6 +104,61 @@ def estimate_sampled(
     return scores
 
 
+def estimate_sampled_map(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    off_q: Optional[torch.Tensor],
+    off_k: Optional[torch.Tensor],
+    block_m: int,
+    block_n: int,
+    keep_m: int,
+    keep_n: int,
+    mask_ratios,
+    text_length: int = 226,
+    mode: str = "topk",
+    min_full_attn_ratio: float = 0.06,
+    compute_tile: int = 32,
+    map_dtype: torch.dtype = torch.int32,
+    sm_scale: Optional[float] = None,
+    return_scores: bool = False,
+):
+    """estimate_sampled + level_map (dense map modes, blocksize = block_n) with the map taken from each row of
+    scores while it is still on chip: the same map, bit for bit, in two launches instead of three.  Returns the
+    map, or (scores, map) with return_scores."""
+    items, m, newtype = _items(mask_ratios, mode)
+    if newtype:
+        raise ValueError("the fused estimator writes dense maps only")
+    if map_dtype not in (torch.int8, torch.int32):
+        raise ValueError("map_dtype must be int8 or int32")
+    _require_gpu(q, k, off_q, off_k)
+    q, k = _bf16_view(q), _bf16_view(k)
+    B, Hq, Lq, D = q.shape
+    Hkv, Lk = k.shape[1], k.shape[2]
+    sm_scale = D ** -0.5 if sm_scale is None else sm_scale
+    Mq, Nk = -(-Lq // block_m), -(-Lk // block_n)
+    for o, H, keep in ((off_q, Hq, keep_m), (off_k, Hkv, keep_n)):
+        if o is not None and (o.dtype != torch.int32 or tuple(o.shape) != (B, H, keep) or not o.is_contiguous()):
+            raise ValueError("sample offsets must be contiguous int32 [B, H, keep]")
+    div = block_n // compute_tile
+    if div < 1:
+        raise ValueError("compute_tile must not exceed blocksize")
+    n = len(items)
+    lv = (ctypes.c_int32 * n)(*[int(i[0]) for i in items])
+    hi = (ctypes.c_double * n)(*[float(i[1][1]) for i in items])
+    tb = (text_length + block_n - 1) // block_n if text_length > 0 else 0
+    scores = torch.empty(B, Hq, Mq, Nk, dtype=torch.float32, device=q.device) if return_scores else None
+    out = torch.empty(B, Hq, Mq, Nk, dtype=map_dtype, device=q.device)
+    ws = torch.empty(lib.psa_estimate_workspace_bytes(B, Hq, Lq, Lk, block_m, block_n, keep_m, keep_n), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        check(
+            lib.psa_estimate_sampled_map(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D,
+                                         block_m, block_n, keep_m, keep_n, float(sm_scale), Mq, Nk, _ptr(out), out.element_size(),
+                                         m, n, lv, hi, div, tb, float(min_full_attn_ratio), _stream(q)),
+            "psa_estimate_sampled_map",
+        )
+    return (scores, out) if return_scores else out
+
+
 # ----------------------------------------------------------------------------- level map
 def _items(mask_ratios, mode: str):
     if mask_ratios is None:
@@ -365,8 +420,8 @@ def psa_layer_fwd(
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     keep_m, keep_n = block_m // 4, block_n // 4
     sm_scale = qb.shape[-1] ** -0.5 if sm_scale is None else float(sm_scale)
-    scores = estimate_sampled(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, sm_scale)
-    mp = level_map(scores, mask_ratios, text_length, mode, blocksize=block_n, compute_tile=tile_n, map_dtype=torch.int8)
+    mp = estimate_sampled_map(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, mask_ratios, text_length, mode,
+                              compute_tile=tile_n, map_dtype=torch.int8, sm_scale=sm_scale)
     if level_cap is not None:
         mp = map_min_cap(mp, level_cap)
     kp, vp = pool_kv(kb, vb, block_n)

@@ -52,3 +52,41 @@ def test_estimate_then_level_map_matches_oracle_map():
     m = ops.level_map(s, ratios, 0, "thresholdbound", blocksize=128, compute_tile=32)
     ref = O.level_map(s.cpu().numpy(), ratios, 0, "thresholdbound", blocksize=128, compute_tile=32)
     assert np.array_equal(m.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("mode", ["topk", "thresholdbound"])
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,L,D,bm,bn,text",
+    [(1, 2, 2, 4096, 128, 128, 128, 0), (2, 2, 1, 1000, 64, 128, 128, 226), (1, 2, 2, 4096, 64, 64, 64, 0), (1, 1, 1, 2000, 128, 128, 32, 0),
+     (1, 3, 3, 1111, 128, 128, 64, 100), (1, 1, 1, 64, 64, 64, 64, 0), (1, 2, 2, 33000, 128, 128, 128, 0)],
+)
+def test_fused_estimate_and_map_equals_the_two_calls(mode, B, Hq, Hkv, L, D, bm, bn, text):
+    """psa_estimate_sampled_map must return exactly the scores of psa_estimate_sampled and exactly the map
+    psa_level_map makes of them (int8 and int32), with and without the scores output."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import sample_offsets
+
+    q, k = rnd(B, Hq, L, D, seed=11).to(dev()), rnd(B, Hkv, L, D, seed=12).to(dev())
+    km, kn = bm // 4, bn // 4
+    oq, ok = sample_offsets(B, Hq, bm, km, 5).to(dev()), sample_offsets(B, Hkv, bn, kn, 6).to(dev())
+    ratios = {1: (0.0, 0.3), 2: (0.3, 0.45), 4: (0.45, 0.6), 8: (0.6, 0.8), 0: (0.8, 1.0)}
+    scores = ops.estimate_sampled(q, k, oq, ok, bm, bn, km, kn)
+    for dt in (torch.int8, torch.int32):
+        ref = ops.level_map(scores, ratios, text, mode, blocksize=bn, compute_tile=min(32, bn), map_dtype=dt)
+        s2, m2 = ops.estimate_sampled_map(q, k, oq, ok, bm, bn, km, kn, ratios, text, mode, compute_tile=min(32, bn), map_dtype=dt,
+                                          return_scores=True)
+        m3 = ops.estimate_sampled_map(q, k, oq, ok, bm, bn, km, kn, ratios, text, mode, compute_tile=min(32, bn), map_dtype=dt)
+        assert torch.equal(s2, scores)
+        assert m2.dtype == dt and torch.equal(m2, ref) and torch.equal(m3, ref)
+
+
+def test_fused_estimate_and_map_errors():
+    from psa_hip import ops
+
+    q, k = rnd(1, 1, 256, 64, seed=1).to(dev()), rnd(1, 1, 256, 64, seed=2).to(dev())
+    with pytest.raises(ValueError):
+        ops.estimate_sampled_map(q, k, None, None, 64, 64, 16, 16, None, 0, "topk")
+    with pytest.raises(ValueError):
+        ops.estimate_sampled_map(q, k, None, None, 64, 64, 16, 16, {1: (0.0, 1.0)}, 0, "topk_newtype")
+    with pytest.raises(ValueError):
+        ops.estimate_sampled_map(q, k, None, None, 64, 64, 16, 16, {1: (0.0, 1.0)}, 0, "nonsense")
