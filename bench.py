@@ -286,19 +286,27 @@ def main():
 
         ncores = os.cpu_count() or 1
         torch.set_num_threads(min(ncores, 32))
+        def cpu_sample(heads, qblocks):
+            qc, kc, vc = (t[:, heads].float().cpu() for t in (q, k, v))
+            mc = mp[:, heads].cpu().numpy().astype("int32")
+            oqc, okc = off_q[:, heads].cpu(), off_k[:, heads].cpu()
+            t0c = time.perf_counter()
+            s_c = O.estimate_sampled(qc, kc, bm, bn, oqc, okc)
+            O.level_map(s_c.numpy(), ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn)
+            t_front = time.perf_counter() - t0c  # pooling is inside blockwalk
+            t1c = time.perf_counter()
+            O.psa_attention_blockwalk(qc, kc, vc, mc, bm, bn, qblocks=qblocks)
+            t_attn = (time.perf_counter() - t1c) * (Mq / len(qblocks))
+            return (t_front + t_attn) * (H / len(heads))
+
+        # a small sample first (two heads, 32 evenly spaced q-blocks, scaled); if the whole layer fits the
+        # budget of a bounded baseline (<= 30 s), time the whole layer instead
         heads = [0, 1] if H >= 2 else [0]
-        qblocks = list(range(0, Mq, max(1, Mq // 32)))[:32]  # 32 evenly spaced q-blocks per sampled head
-        qc, kc, vc = (t[:, heads].float().cpu() for t in (q, k, v))
-        mc = mp[:, heads].cpu().numpy().astype("int32")
-        oqc, okc = off_q[:, heads].cpu(), off_k[:, heads].cpu()
-        t0c = time.perf_counter()
-        s_c = O.estimate_sampled(qc, kc, bm, bn, oqc, okc)
-        O.level_map(s_c.numpy(), ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn)
-        t_front = time.perf_counter() - t0c  # pooling is inside blockwalk
-        t1c = time.perf_counter()
-        O.psa_attention_blockwalk(qc, kc, vc, mc, bm, bn, qblocks=qblocks)
-        t_attn = (time.perf_counter() - t1c) * (Mq / len(qblocks))
-        cpu_s_per_layer = (t_front + t_attn) * (H / len(heads))
+        qblocks = list(range(0, Mq, max(1, Mq // 32)))[:32]
+        cpu_s_per_layer = cpu_sample(heads, qblocks)
+        if cpu_s_per_layer <= 30.0:
+            heads, qblocks = list(range(H)), list(range(Mq))
+            cpu_s_per_layer = cpu_sample(heads, qblocks)
         cpu = {
             "value": round(dense_flops / cpu_s_per_layer / 1e12, 5),
             "unit": "TFLOP/s (effective)",
@@ -306,8 +314,10 @@ def main():
             "cores": torch.get_num_threads(),
             "host_cpus": ncores,
             "kind": "port",
-            "sample": "heads %s of %d in fp32: full estimate + level map, attention on %d of %d q-blocks scaled to all; "
-                      "then scaled by H/%d" % (heads, H, len(qblocks), Mq, len(heads)),
+            "sample": ("the whole layer in fp32: all %d heads, all %d q-blocks (estimate + level map + attention)" % (H, Mq))
+            if len(heads) == H and len(qblocks) == Mq else
+            ("heads %s of %d in fp32: full estimate + level map, attention on %d of %d q-blocks scaled to all; "
+             "then scaled by H/%d" % (heads, H, len(qblocks), Mq, len(heads))),
         }
 
     if args.copy_calib:
