@@ -412,10 +412,10 @@ def psa_layer_fwd(
     return_map: bool = False,
     text_length: int = 0,
 ):
-    """estimate -> level map -> pooled K/V -> sparse attention, non-causal, no gradient: the four stages
-    on the current stream with a dense int8 level map in between (no index-list round trip).  Running the
-    pooling pass on a second stream beside the level-map kernel was measured and gains nothing: the
-    level-map launch already occupies every wave slot of the chip."""
+    """estimate (+ level map, in the estimator's reduction kernel) -> pooled K/V -> sparse attention, non-causal,
+    no gradient: all on the current stream with a dense int8 level map in between (no index-list round trip).
+    Running the pooling pass on a second stream beside the estimator or the level map was measured and gains
+    nothing: those launches occupy every register and wave slot of the chip."""
     _require_gpu(q, k, v)
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     keep_m, keep_n = block_m // 4, block_n // 4
