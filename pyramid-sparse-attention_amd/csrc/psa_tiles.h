@@ -284,7 +284,9 @@ __device__ __forceinline__ void lt_tile_src(const KvSource& kv, const u32x2* tde
   const int cnt = d1 >> 16;
   const uint16_t* lids = ids + (d1 & 0xffff);
   const int sbs_log2 = kv.bn_log2 - lv;
-  const int lm1 = lv > 0 ? lv - 1 : 0;
+  // max(lv - 1, 0) from a table in a constant: a saturating subtraction would be a vector instruction and drag the
+  // 64-bit offset arithmetic below (and the copy base pointers) from the scalar to the vector unit
+  const int lm1 = (0x2100 >> (4 * lv)) & 3;
   const int64_t pool_off = (kv.BHkv * (kv.npad - (kv.npad >> lm1)) + kv.bhk * (kv.npad >> lv)) * (D * 2);
   a.kbase = lv == 0 ? kv.k0 : kv.kp + pool_off;
   a.vbase = lv == 0 ? kv.v0 : kv.vp + pool_off;
