@@ -88,8 +88,8 @@ __global__ __launch_bounds__(X_WAVES * 64, 1) void psa_xattn_gemm_kernel(XParams
   const char* qb = (const char*)(p.q + b * p.q_sb + h * p.q_sh);
   const char* kb = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
   const uint32_t q_strb = (uint32_t)p.q_sl * 2u, k_strb = (uint32_t)p.k_sl * 2u;
-  const int dchunks = p.D / KC;
-  const int stages = S * dchunks;
+  const int dc_log2 = p.D == 2 * KC ? 1 : 0;  // 64-channel chunks per row: 1 (D = 64) or 2 (D = 128)
+  const int stages = S << dc_log2;
 
   // copies: wave w moves the 16-row groups w*X_GPW .. of a stage (group g: tile g/4, rows 16*(g%4)..), a lane
   // the RPL consecutive rows frow.. of each group; a row is one strided index (S tokens apart in memory)
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(X_WAVES * 64, 1) void psa_xattn_gemm_kernel(XParams
   // copy instruction `piece` (0 .. X_GPW * RPL - 1) of stage st
   auto issue_piece = [&](int st, int piece) __attribute__((always_inline)) {
     const int j = piece / RPL, n = piece % RPL;
-    const int i = st / dchunks, dc = st % dchunks;
+    const int i = st >> dc_log2, dc = st & ((1 << dc_log2) - 1);  // (shifts: a division here would run on the vector unit and take the base pointers with it)
     unsigned char* dst = smem + (st & 1) * X_STAGE;
     const int g = wave * X_GPW + j, tile = g >> 2;
     const bool is_q = tile < X_QT;
