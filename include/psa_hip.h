@@ -100,7 +100,9 @@ int psa_level_map(const float* scores, void* map_out, int map_elem_bytes, int32_
 /* psa_estimate_sampled followed by psa_level_map (dense map only) in two launches instead of three: the kernel that
  * reduces the estimator's workspace to a row of scores goes on to rank that row while it is still in LDS.  The map
  * [B, Hq, out_rows, out_cols] is the one psa_level_map computes from the scores psa_estimate_sampled returns, bit for
- * bit; `scores` may be NULL when only the map is wanted.  Arguments as in the two functions (Nk = out_cols).
+ * bit; `scores` may be NULL when only the map is wanted, except for maps wider than about 5000 columns (the row and
+ * the ranking scratch then exceed LDS together and the function runs the two kernels one after the other, which needs
+ * the scores buffer: PSA_ERR_ARG without it).  Arguments as in the two functions (Nk = out_cols).
  * Replaces the same reference code as they do (attn_with_pooling_optimized + transfer_attn_to_mask as called from
  * reference src/psa_triton/attention.py:178-235). */
 int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k,

@@ -314,7 +314,7 @@ __global__ __launch_bounds__(256) void psa_est_reduce_map_kernel(EstParams p, Le
 }
 
 template <int D>
-int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp) {
+int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp, bool* map_done) {
   const int rows_needed = p.out_rows << p.keep_m_log2;
   dim3 grid((unsigned)((rows_needed + 255) / 256), (unsigned)(B * p.Hq));
   // 256-row workgroups: cut the key range until about 3 workgroups per CU exist (the kernel's occupancy),
@@ -338,11 +338,19 @@ int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp
   }
   const size_t lm_bytes = (level_map_lds_bytes(lp->Nk) + 15) & ~(size_t)15;
   const size_t shmem = lm_bytes + (size_t)p.n_d * sizeof(float);
+  if (shmem > 150 * 1024) {
+    // very wide maps: the row of scores and the level-map scratch do not fit into LDS together - two kernels
+    PSA_REQUIRE(p.scores != nullptr, PSA_ERR_ARG, "psa_estimate_sampled_map: maps of %d columns need the scores buffer", lp->Nk);
+    hipLaunchKernelGGL(psa_est_reduce_kernel, rgrid, dim3(256), (size_t)p.n_d * sizeof(float), stream, p);
+    *map_done = false;  // the caller finishes with psa_level_map on the scores
+    return psa_check_launch("psa_estimate_sampled_map (reduction)");
+  }
   if (shmem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)psa_est_reduce_map_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_estimate_sampled_map: cannot reserve %zu bytes of LDS", shmem);
   }
   hipLaunchKernelGGL(psa_est_reduce_map_kernel, rgrid, dim3(256), shmem, stream, p, *lp, (int)lm_bytes);
+  *map_done = true;
   return psa_check_launch("psa_estimate_sampled_map (reduction + level map)");
 }
 
@@ -373,7 +381,7 @@ extern "C" int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, i
 namespace {
 int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores, void* workspace, int B, int Hq,
             int Hkv, int Lq, int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale, int out_rows,
-            int out_cols, LevelMapParams* lp, psa_stream_t stream) {
+            int out_cols, LevelMapParams* lp, bool* map_done, psa_stream_t stream) {
   PSA_REQUIRE(q.ptr && k.ptr && (scores || lp) && workspace, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Lq > 0 && Lk > 0, PSA_ERR_ARG, "psa_estimate_sampled: sizes must be positive");
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_estimate_sampled: Hq must be a multiple of Hkv");
@@ -406,7 +414,7 @@ int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* o
     PSA_REQUIRE(lp->Nk == out_cols, PSA_ERR_ARG, "psa_estimate_sampled_map: the map has %d columns, the scores %d", lp->Nk, out_cols);
     lp->scores = nullptr;
   }
-  return D == 128 ? launch_est<128>(p, B, (hipStream_t)stream, lp) : launch_est<64>(p, B, (hipStream_t)stream, lp);
+  return D == 128 ? launch_est<128>(p, B, (hipStream_t)stream, lp, map_done) : launch_est<64>(p, B, (hipStream_t)stream, lp, map_done);
 }
 }  // namespace
 
@@ -414,8 +422,9 @@ extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t*
                                     void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
                                     int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
   PSA_REQUIRE(scores, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
+  bool unused = false;
   return est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale, out_rows,
-                 out_cols, nullptr, stream);
+                 out_cols, nullptr, &unused, stream);
 }
 
 extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
@@ -430,6 +439,10 @@ extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int3
   const int rc = level_map_fill_params(lp, out_cols, mode, n_items, item_level, item_hi, align_div, text_blocks, min_full_attn_ratio);
   if (rc != PSA_OK) return rc;
   lp.map_out = map_out; lp.map_elem = map_elem_bytes;
-  return est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale, out_rows,
-                 out_cols, &lp, stream);
+  bool map_done = false;
+  const int rc2 = est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
+                          out_rows, out_cols, &lp, &map_done, stream);
+  if (rc2 != PSA_OK || map_done) return rc2;
+  return psa_level_map(scores, map_out, map_elem_bytes, nullptr, (int64_t)B * Hq * out_rows, out_cols, mode, n_items, item_level, item_hi,
+                       align_div, text_blocks, min_full_attn_ratio, stream);
 }

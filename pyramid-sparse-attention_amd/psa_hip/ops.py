@@ -146,7 +146,8 @@ def estimate_sampled_map(
     lv = (ctypes.c_int32 * n)(*[int(i[0]) for i in items])
     hi = (ctypes.c_double * n)(*[float(i[1][1]) for i in items])
     tb = (text_length + block_n - 1) // block_n if text_length > 0 else 0
-    scores = torch.empty(B, Hq, Mq, Nk, dtype=torch.float32, device=q.device) if return_scores else None
+    # (maps wider than about 5000 columns do not fit the fused kernel's LDS: the library then needs the scores buffer)
+    scores = torch.empty(B, Hq, Mq, Nk, dtype=torch.float32, device=q.device) if (return_scores or Nk > 4096) else None
     out = torch.empty(B, Hq, Mq, Nk, dtype=map_dtype, device=q.device)
     ws = torch.empty(lib.psa_estimate_workspace_bytes(B, Hq, Lq, Lk, block_m, block_n, keep_m, keep_n), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

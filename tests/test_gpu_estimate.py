@@ -90,3 +90,16 @@ def test_fused_estimate_and_map_errors():
         ops.estimate_sampled_map(q, k, None, None, 64, 64, 16, 16, {1: (0.0, 1.0)}, 0, "topk_newtype")
     with pytest.raises(ValueError):
         ops.estimate_sampled_map(q, k, None, None, 64, 64, 16, 16, {1: (0.0, 1.0)}, 0, "nonsense")
+
+
+def test_fused_estimate_and_map_very_wide_rows_fall_back_to_two_kernels():
+    """6000 key blocks: the row of scores and the level-map scratch exceed LDS together; same results by two kernels."""
+    from psa_hip import ops
+
+    L, bm, bn = 192000, 128, 32
+    q, k = rnd(1, 1, L, 64, seed=21).to(dev()), rnd(1, 1, L, 64, seed=22).to(dev())
+    ratios = {1: (0.0, 0.05), 2: (0.05, 0.1), 4: (0.1, 0.2), 8: (0.2, 0.4), 0: (0.4, 1.0)}
+    scores = ops.estimate_sampled(q, k, None, None, bm, bn, 32, 8)
+    ref = ops.level_map(scores, ratios, 0, "thresholdbound", blocksize=bn, compute_tile=32, map_dtype=torch.int8)
+    got = ops.estimate_sampled_map(q, k, None, None, bm, bn, 32, 8, ratios, 0, "thresholdbound", compute_tile=32, map_dtype=torch.int8)
+    assert got.shape == (1, 1, 1500, 6000) and torch.equal(got, ref)
