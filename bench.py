@@ -21,7 +21,6 @@ sys.path.insert(0, PKG)
 
 METRIC = "PSA attn ms/layer + effective TFLOPS (% bf16 MFMA peak) at Wan2.1-1.3B shape, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-SUSTAINED_BF16_TFLOPS = 1800.0  # measured: pure MFMA loop, random bf16 operands, 30-60 ms, one MI355X
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
@@ -256,6 +255,31 @@ def main():
         t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
         t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
 
+    # ---- what the chip sustains on a register-only MFMA loop, measured now (constant and random operands) ----
+    def mfma_probe(random_operands):
+        from psa_hip._lib import lib as _l
+        import ctypes as _ct
+        props = torch.cuda.get_device_properties(dev)
+        sink = torch.zeros(256, dtype=torch.float32, device=dev)
+        clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+        flops = _ct.c_double(0.0)
+        wgs, iters = props.multi_processor_count * 2, 40000  # 2 waves per SIMD, about 30-45 ms
+        best = None
+        for _ in range(2):  # the first launch also ramps the clocks down to their sustained level
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = _l.psa_probe_mfma(wgs, iters, int(random_operands), _ct.c_void_p(sink.data_ptr()), _ct.c_void_p(clocks.data_ptr()),
+                                   _ct.byref(flops), _ct.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0
+            b_.record()
+            torch.cuda.synchronize()
+            c = clocks.cpu()
+            best = {"tflops": round(flops.value / (a.elapsed_time(b_) * 1e-3) / 1e12, 1),
+                    "core_clock_ghz": round(float(c[1]) / max(float(c[0]), 1.0) / 10.0, 3)}
+        return best
+
+    probe_const, probe_rand = mfma_probe(False), mfma_probe(True)
+
     pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
 
@@ -272,10 +296,12 @@ def main():
         "flops_per_launch": exec_flops,
         "avg_launch_ms": round(t_fwd_avg, 4),
         "launch_includes": "the forward kernel and its two row-ordering launches (about 9 us together)",
-        # a register-only loop of independent bf16 MFMAs with random operands sustains this much on the same chip
-        # (power management); with constant operands it reaches 2460
-        "sustained_mfma_tflops_random_operands": SUSTAINED_BF16_TFLOPS,
-        "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / SUSTAINED_BF16_TFLOPS, 4),
+        # what a register-only loop of independent bf16 MFMAs sustains on this chip right now (psa_probe_mfma, 2 waves
+        # per SIMD, 30-45 ms): the clock falls under a dense MFMA stream, further when the operands toggle
+        "mfma_probe_constant_operands": probe_const,
+        "mfma_probe_random_operands": probe_rand,
+        "sustained_mfma_tflops_random_operands": probe_rand["tflops"],
+        "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_rand["tflops"], 4),
     }
 
     # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------

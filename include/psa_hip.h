@@ -174,6 +174,14 @@ int psa_gather_rows(const psa_tensor4* src, const psa_tensor4* dst, const int* h
 int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk, int causal,
                 float* density_out, psa_stream_t stream);
 
+/* Diagnostic, no counterpart in the reference (bench.py uses it to put the measured MFMA utilisation of the attention
+ * kernels next to what the chip sustains): `workgroups` x 4 waves each issue iters x 16 independent bf16 32x32x16 MFMAs
+ * from registers (random_operands != 0: pseudo-random values, else one constant).  sink: >= 256 floats of device memory
+ * (never written in practice), clocks: 2 x int64 of device memory = ticks of the constant 100 MHz counter and of the
+ * core clock counter over the loop of the first wave, *flops (host, may be NULL) = floating-point operations issued. */
+int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,
+                   psa_stream_t stream);
+
 /* Sparse attention forward from a level map.  out [B, Hq, L, D] bf16; lse (may be NULL)
  * [B, Hq, L] fp32 = natural-log softmax denominator incl. the +ln(level) bias; map == NULL means
  * dense attention (every pair at level 1; k_pool/v_pool may then be NULL).  K/V have Hkv heads,
