@@ -278,7 +278,7 @@ def main():
                     "core_clock_ghz": round(float(c[1]) / max(float(c[0]), 1.0) / 10.0, 3)}
         return best
 
-    probe_const, probe_rand = mfma_probe(False), mfma_probe(True)
+    probe_const, probe_rand, probe_lds = mfma_probe(0), mfma_probe(1), mfma_probe(2)
 
     pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
@@ -300,8 +300,10 @@ def main():
         # per SIMD, 30-45 ms): the clock falls under a dense MFMA stream, further when the operands toggle
         "mfma_probe_constant_operands": probe_const,
         "mfma_probe_random_operands": probe_rand,
+        "mfma_probe_random_operands_a_from_lds": probe_lds,
         "sustained_mfma_tflops_random_operands": probe_rand["tflops"],
         "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_rand["tflops"], 4),
+        "frac_of_sustained_a_from_lds": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_lds["tflops"], 4),
     }
 
     # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------

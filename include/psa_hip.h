@@ -176,7 +176,8 @@ int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk,
 
 /* Diagnostic, no counterpart in the reference (bench.py uses it to put the measured MFMA utilisation of the attention
  * kernels next to what the chip sustains): `workgroups` x 4 waves each issue iters x 16 independent bf16 32x32x16 MFMAs
- * from registers (random_operands != 0: pseudo-random values, else one constant).  sink: >= 256 floats of device memory
+ * from registers (random_operands 0: one constant, 1: pseudo-random values, 2: pseudo-random and the A operand of every
+ * MFMA re-read from LDS).  sink: >= 256 floats of device memory
  * (never written in practice), clocks: 2 x int64 of device memory = ticks of the constant 100 MHz counter and of the
  * core clock counter over the loop of the first wave, *flops (host, may be NULL) = floating-point operations issued. */
 int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,

@@ -4,7 +4,8 @@
 // (power management), and how far depends on how much the operands toggle.  bench.py runs this next to the
 // attention kernels so that their MFMA utilisation can be read against what the same chip sustains at that moment.
 // Every wave keeps 4 A and 4 B operands in registers and issues iters * 4 independent 32x32x16 MFMAs on 4
-// accumulators; nothing touches LDS or memory inside the loop.
+// accumulators; nothing touches LDS or memory inside the loop (modes 0 and 1), or every MFMA takes its A operand from
+// LDS (mode 2).
 #include "psa_common.h"
 
 namespace {
@@ -27,12 +28,40 @@ __global__ __launch_bounds__(256) void psa_probe_mfma_kernel(int iters, int rand
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int i = 0; i < 16; ++i) c[j][i] = 0.f;
+  // mode 2: the A operand of every MFMA is read from LDS (one 128-bit read per MFMA, the ratio of the attention
+  // kernels), 16 KiB of pseudo-random bf16 per wave slot, conflict-free addresses
+  __shared__ __align__(16) unsigned char lds[4 * 16 * 1024];
+  if (random_operands == 2) {
+    uint32_t* w = (uint32_t*)lds;
+    for (int i = threadIdx.x; i < (int)sizeof(lds) / 4; i += 256) {
+      r = r * 1664525u + 1013904223u;
+      const uint32_t lo = __builtin_bit_cast(uint16_t, (bf16_t)(((int)(r >> 8) % 2001 - 1000) * (1.0f / 64000.f)));
+      r = r * 1664525u + 1013904223u;
+      const uint32_t hi = __builtin_bit_cast(uint16_t, (bf16_t)(((int)(r >> 8) % 2001 - 1000) * (1.0f / 64000.f)));
+      w[i] = lo | (hi << 16);
+    }
+    __syncthreads();
+  }
+  const unsigned char* my = lds + (threadIdx.x >> 6) * 16 * 1024 + (threadIdx.x & 63) * 16;
   const long long w0 = wall_clock64(), c0 = clock64();
-  for (int it = 0; it < iters; ++it) {
+  if (random_operands == 2) {
+    for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 4; ++u) {
+        bf16x8 al[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], b[(j + u) & 3], c[j], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) al[j] = *(const bf16x8*)(my + (((it + u) & 3) * 4 + j) * 1024);  // varies with `it`: stays in the loop
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[j], b[(j + u) & 3], c[j], 0, 0, 0);
+      }
+    }
+  } else {
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], b[(j + u) & 3], c[j], 0, 0, 0);
+    }
   }
   const long long w1 = wall_clock64(), c1 = clock64();
   float s = 0.f;
