@@ -159,6 +159,41 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
     }
 
 
+def run_probe(torch, dev):
+    """The synthetic attention-shaped loop of psa_probe_attention, 2 workgroups per CU, about 40-60 ms per variant."""
+    import ctypes as ct
+
+    from psa_hip._lib import lib
+
+    wgs = torch.cuda.get_device_properties(dev).multi_processor_count * 2
+    iters = 25000
+    sink = torch.zeros(256, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    src = torch.zeros(wgs * 256 * 1024, dtype=torch.uint8, device=dev)
+    flops = ct.c_double(0.0)
+    names = {0: "base: 32 MFMAs (A from LDS) + minimal softmax per tile and wave", 1: "+ workgroup barrier per tile",
+             8: "+ PV operands through the transposing LDS load", 4: "+ 8 global->LDS copies per wave and tile (source in L2)",
+             20: "+ the same copies from the fabric (64 KiB per wave)", 2: "+ 100 more vector instructions per tile",
+             15: "barrier + transposing loads + copies (L2) + 100 vector instructions"}
+    out = []
+    for feat in (0, 1, 8, 4, 20, 2, 15):
+        res = None
+        for _ in range(2):  # the first launch settles the clocks
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = lib.psa_probe_attention(wgs, iters, feat, ct.c_void_p(src.data_ptr()), ct.c_void_p(sink.data_ptr()),
+                                         ct.c_void_p(clocks.data_ptr()), ct.byref(flops), ct.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b)
+            c = clocks.cpu()
+            res = {"features": feat, "what": names[feat], "tflops": round(flops.value / (ms * 1e-3) / 1e12, 1),
+                   "ns_per_tile_and_simd": round(ms * 1e6 / iters / 2, 1), "core_clock_ghz": round(float(c[1]) / max(float(c[0]), 1.0) / 10.0, 3)}
+        out.append(res)
+    return {"probe": "attention-shaped synthetic loop, 4 waves per workgroup, 2 workgroups per CU, free-running", "variants": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,6 +206,9 @@ def main():
     ap.add_argument("--copy-calib", action="store_true",
                     help="after the run, stream 1 GiB through a plain elementwise kernel (reads 1 GiB, writes 1 GiB): "
                          "under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its reading calibrates the counters")
+    ap.add_argument("--probe", action="store_true",
+                    help="instead of the workload, run the synthetic attention-shaped loop (psa_probe_attention) with one feature of "
+                         "the real kernels at a time and print what the chip sustains for each")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by (batch, head) with no exchange, "
@@ -189,6 +227,9 @@ def main():
     w = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.probe:
+        print(json.dumps(run_probe(torch, dev)))
+        return
     if w.get("kind") in ("train", "causal"):
         print(json.dumps(run_other(args, w, torch, ops, make_qkv, sample_offsets, dev)))
         return

@@ -183,6 +183,15 @@ int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk,
 int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,
                    psa_stream_t stream);
 
+/* Diagnostic, no counterpart in the reference (bench.py --probe): an attention-shaped loop on synthetic data - per tile
+ * and wave 16 QK MFMAs with one operand from LDS, a minimal softmax over the 32 logits, 16 PV MFMAs; 4 waves per workgroup,
+ * free-running.  `features` adds what the real kernels have, one at a time: 1 = a workgroup barrier per tile, 2 = 100 more
+ * vector instructions per tile, 4 = 8 global->LDS copies per wave and tile from an L2-resident source, 8 = PV operands
+ * through the transposing LDS load, 15 = all of them, 20 = the copies of 4 from a private 64 KiB per wave (fabric-bound).
+ * copy_source: workgroups * 256 KiB of device memory; sink, clocks, flops as in psa_probe_mfma. */
+int psa_probe_attention(int workgroups, int iters, int features, const void* copy_source, float* sink, int64_t* clocks,
+                        double* flops, psa_stream_t stream);
+
 /* Sparse attention forward from a level map.  out [B, Hq, L, D] bf16; lse (may be NULL)
  * [B, Hq, L] fp32 = natural-log softmax denominator incl. the +ln(level) bias; map == NULL means
  * dense attention (every pair at level 1; k_pool/v_pool may then be NULL).  K/V have Hkv heads,

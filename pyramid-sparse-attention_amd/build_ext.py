@@ -30,6 +30,7 @@ FLAGS = [
 FILE_FLAGS = {
     "psa_fwd.hip": ["-fno-honor-nans"],
     "psa_estimate.hip": ["-fno-honor-nans"],
+    "psa_probe.hip": ["-fno-honor-nans"],  # the synthetic loop is compiled like the forward kernel it models
 }
 
 

@@ -76,6 +76,113 @@ __global__ __launch_bounds__(256) void psa_probe_mfma_kernel(int iters, int rand
   }
 }
 
+
+// Attention-shaped loop: per tile and wave 16 QK MFMAs (A operand from LDS), a minimal softmax on the 32 logits (max
+// chain, fma + exp2 + add per logit, bf16 packing), 16 PV MFMAs; 4 waves per workgroup, 2 workgroups per CU,
+// free-running.  FLAGS add one feature of the real kernels each: 1 = workgroup barrier per tile, 2 = 100 more vector
+// instructions per tile, 4 = 8 global->LDS copies per wave and tile and vmcnt(0) before the barrier, 8 = PV operands
+// through the transposing LDS load; L2RES: the copies read a source that stays in L2 instead of one per wave.
+template <int FLAGS, int L2RES>
+__global__ __launch_bounds__(256, 2) void psa_probe_attn_kernel(int iters, const char* gsrc, float* sink, long long* clocks) {
+  __shared__ __align__(16) unsigned char lds[72 * 1024];  // 64 KiB of operands + 8 KiB copy target
+  uint32_t r = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+  for (int i = threadIdx.x; i < 64 * 1024 / 4; i += 256) {
+    r = r * 1664525u + 1013904223u;
+    const float f0 = ((int)(r >> 8) % 2001 - 1000) * (1.0f / 2000.f);
+    r = r * 1664525u + 1013904223u;
+    const float f1 = ((int)(r >> 8) % 2001 - 1000) * (1.0f / 2000.f);
+    ((uint32_t*)lds)[i] = pack_bf16x2(f0, f1);
+  }
+  __syncthreads();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const unsigned char* my = lds + wave * 16 * 1024 + lane * 16;
+  const unsigned char* my8 = lds + wave * 16 * 1024 + lane * 8;
+  bf16x8 q[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) q[j] = *(const bf16x8*)(my + j * 1024);
+  f32x16 acc[4], s[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  uint32_t pk[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) pk[i] = 0;
+  float m_run = 0.f, l_run = 0.f, junk = 1.0f;
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const uint32_t copy_dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)(lds + 64 * 1024) + wave * 2048;
+  const char* gs = gsrc + ((size_t)(L2RES ? (blockIdx.x & 15) : blockIdx.x) * 4 + wave) * 65536;
+  const long long w0 = wall_clock64(), c0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+    if (FLAGS & 4) {
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {
+        const uint32_t voff = (uint32_t)(((it * 8 + n) & 63) * 1024 + lane * 16);
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(copy_dst + (n & 1) * 1024);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(gs) : "memory");
+      }
+    }
+    s[0] = zero;
+    s[1] = zero;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      const bf16x8 a0 = *(const bf16x8*)(my + (((it + kk) & 7) * 2) * 1024), a1 = *(const bf16x8*)(my + (((it + kk) & 7) * 2 + 1) * 1024);
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q[kk], s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q[kk], s[1], 0, 0, 0);
+    }
+    {
+      float mx = s[0][0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
+      m_run = fmaxf(m_run, mx * 0.001f);
+      const float nb = -m_run;
+      float lsum = 0.f;
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = fast_exp2(__builtin_fmaf(s[c][i], 0.01f, nb));
+          const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], 0.01f, nb));
+          pk[c * 8 + (i >> 1)] = pack_bf16x2(p0, p1);
+          lsum += p0 + p1;
+        }
+      l_run = l_run * 0.999f + lsum;
+      if (FLAGS & 2) {
+#pragma unroll
+        for (int i = 0; i < 100; ++i) junk = __builtin_fmaf(junk, 1.0001f, s[i & 1][i & 15]);
+      }
+    }
+#pragma unroll
+    for (int st = 0; st < 16; ++st) {
+      bf16x8 a;
+      if (FLAGS & 8) {
+        typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4_ptr;
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(my8 + ((it + st) & 15) * 1024)));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(my8 + ((it + st) & 15) * 1024 + 512)));
+        u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+        a = __builtin_bit_cast(bf16x8, w);
+      } else {
+        a = *(const bf16x8*)(my + ((it + st) & 15) * 1024);
+      }
+      u32x4 bw = {pk[(st >> 2) * 4], pk[(st >> 2) * 4 + 1], pk[(st >> 2) * 4 + 2], pk[(st >> 2) * 4 + 3]};
+      acc[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, __builtin_bit_cast(bf16x8, bw), acc[st & 3], 0, 0, 0);
+    }
+    if (FLAGS & 4) __builtin_amdgcn_s_waitcnt(0x0f70);
+    if (FLAGS & 1) __syncthreads();
+  }
+  const long long w1 = wall_clock64(), c1 = clock64();
+  float t = l_run + junk;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += acc[j][i];
+  if (t == 1.2345f) sink[threadIdx.x] = t;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    clocks[0] = w1 - w0;
+    clocks[1] = c1 - c0;
+  }
+}
+
 }  // namespace
 
 extern "C" int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,
@@ -85,4 +192,25 @@ extern "C" int psa_probe_mfma(int workgroups, int iters, int random_operands, fl
                      (long long*)clocks);
   if (flops) *flops = (double)workgroups * 4.0 * iters * 16.0 * (2.0 * 32 * 32 * 16);  // 4 waves x 16 MFMAs per iteration
   return psa_check_launch("psa_probe_mfma");
+}
+
+extern "C" int psa_probe_attention(int workgroups, int iters, int features, const void* copy_source, float* sink, int64_t* clocks,
+                                   double* flops, psa_stream_t stream) {
+  PSA_REQUIRE(workgroups > 0 && iters > 0 && sink && clocks && copy_source, PSA_ERR_ARG, "psa_probe_attention: bad arguments");
+  const dim3 g((unsigned)workgroups), b(256);
+  hipStream_t st = (hipStream_t)stream;
+  const char* src = (const char*)copy_source;
+  long long* ck = (long long*)clocks;
+  switch (features) {
+    case 0: hipLaunchKernelGGL((psa_probe_attn_kernel<0, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 1: hipLaunchKernelGGL((psa_probe_attn_kernel<1, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 2: hipLaunchKernelGGL((psa_probe_attn_kernel<2, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 4: hipLaunchKernelGGL((psa_probe_attn_kernel<4, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 8: hipLaunchKernelGGL((psa_probe_attn_kernel<8, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 15: hipLaunchKernelGGL((psa_probe_attn_kernel<15, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 16 + 4: hipLaunchKernelGGL((psa_probe_attn_kernel<4, 0>), g, b, 0, st, iters, src, sink, ck); break;
+    default: PSA_REQUIRE(false, PSA_ERR_ARG, "psa_probe_attention: features must be 0, 1, 2, 4, 8, 15 or 20");
+  }
+  if (flops) *flops = (double)workgroups * 4.0 * iters * 32.0 * (2.0 * 32 * 32 * 16);  // 4 waves x 32 MFMAs per tile
+  return psa_check_launch("psa_probe_attention");
 }
