@@ -174,9 +174,9 @@ def run_probe(torch, dev):
     names = {0: "base: 32 MFMAs (A from LDS) + minimal softmax per tile and wave", 1: "+ workgroup barrier per tile",
              8: "+ PV operands through the transposing LDS load", 4: "+ 8 global->LDS copies per wave and tile (source in L2)",
              20: "+ the same copies from the fabric (64 KiB per wave)", 2: "+ 100 more vector instructions per tile",
-             15: "barrier + transposing loads + copies (L2) + 100 vector instructions"}
+             13: "barrier + transposing loads + copies (L2)", 15: "barrier + transposing loads + copies (L2) + 100 vector instructions"}
     out = []
-    for feat in (0, 1, 8, 4, 20, 2, 15):
+    for feat in (0, 1, 8, 4, 20, 2, 13, 15):
         res = None
         for _ in range(2):  # the first launch settles the clocks
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

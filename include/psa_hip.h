@@ -187,7 +187,7 @@ int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, 
  * and wave 16 QK MFMAs with one operand from LDS, a minimal softmax over the 32 logits, 16 PV MFMAs; 4 waves per workgroup,
  * free-running.  `features` adds what the real kernels have, one at a time: 1 = a workgroup barrier per tile, 2 = 100 more
  * vector instructions per tile, 4 = 8 global->LDS copies per wave and tile from an L2-resident source, 8 = PV operands
- * through the transposing LDS load, 15 = all of them, 20 = the copies of 4 from a private 64 KiB per wave (fabric-bound).
+ * through the transposing LDS load, 13 = 1 + 4 + 8, 15 = all of them, 20 = the copies of 4 from a private 64 KiB per wave (fabric-bound).
  * copy_source: workgroups * 256 KiB of device memory; sink, clocks, flops as in psa_probe_mfma. */
 int psa_probe_attention(int workgroups, int iters, int features, const void* copy_source, float* sink, int64_t* clocks,
                         double* flops, psa_stream_t stream);

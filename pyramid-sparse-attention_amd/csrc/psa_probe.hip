@@ -207,9 +207,10 @@ extern "C" int psa_probe_attention(int workgroups, int iters, int features, cons
     case 2: hipLaunchKernelGGL((psa_probe_attn_kernel<2, 1>), g, b, 0, st, iters, src, sink, ck); break;
     case 4: hipLaunchKernelGGL((psa_probe_attn_kernel<4, 1>), g, b, 0, st, iters, src, sink, ck); break;
     case 8: hipLaunchKernelGGL((psa_probe_attn_kernel<8, 1>), g, b, 0, st, iters, src, sink, ck); break;
+    case 13: hipLaunchKernelGGL((psa_probe_attn_kernel<13, 1>), g, b, 0, st, iters, src, sink, ck); break;
     case 15: hipLaunchKernelGGL((psa_probe_attn_kernel<15, 1>), g, b, 0, st, iters, src, sink, ck); break;
     case 16 + 4: hipLaunchKernelGGL((psa_probe_attn_kernel<4, 0>), g, b, 0, st, iters, src, sink, ck); break;
-    default: PSA_REQUIRE(false, PSA_ERR_ARG, "psa_probe_attention: features must be 0, 1, 2, 4, 8, 15 or 20");
+    default: PSA_REQUIRE(false, PSA_ERR_ARG, "psa_probe_attention: features must be 0, 1, 2, 4, 8, 13, 15 or 20");
   }
   if (flops) *flops = (double)workgroups * 4.0 * iters * 32.0 * (2.0 * 32 * 32 * 16);  // 4 waves x 32 MFMAs per tile
   return psa_check_launch("psa_probe_attention");

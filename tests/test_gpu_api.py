@@ -198,7 +198,7 @@ def test_mfma_probe_runs_and_reports_clocks():
     assert lib.psa_probe_mfma(0, 500, 0, ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(clocks.data_ptr()), None, None) != 0
 
 
-@pytest.mark.parametrize("features", [0, 1, 2, 4, 8, 15, 20])
+@pytest.mark.parametrize("features", [0, 1, 2, 4, 8, 13, 15, 20])
 def test_attention_probe_variants_run(features):
     """bench.py --probe: every variant of the synthetic attention-shaped loop launches, finishes and counts its flops."""
     import ctypes
