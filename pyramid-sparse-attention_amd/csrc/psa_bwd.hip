@@ -317,16 +317,17 @@ __global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int s
   }
 }
 
-// one workgroup: counting sort of all workgroup ids by decreasing cost
-__global__ __launch_bounds__(256) void psa_bwd_colsort_kernel(const int32_t* cost, int total, int32_t* order) {
+// one workgroup of 1024 threads: counting sort of all workgroup ids by decreasing cost
+constexpr int COLSORT_NT = 1024;
+__global__ __launch_bounds__(COLSORT_NT) void psa_bwd_colsort_kernel(const int32_t* cost, int total, int32_t* order) {
   __shared__ int hist[COL_BINS];
-  __shared__ int part[256];
+  __shared__ int part[COLSORT_NT];
   const int tid = threadIdx.x;
-  for (int i = tid; i < COL_BINS; i += 256) hist[i] = 0;
+  for (int i = tid; i < COL_BINS; i += COLSORT_NT) hist[i] = 0;
   __syncthreads();
-  for (int i = tid; i < total; i += 256) atomicAdd(&hist[cost[i]], 1);
+  for (int i = tid; i < total; i += COLSORT_NT) atomicAdd(&hist[cost[i]], 1);
   __syncthreads();
-  constexpr int PER = COL_BINS / 256;  // thread i owns the bins COL_BINS-1-PER*i .. COL_BINS-PER-PER*i
+  constexpr int PER = COL_BINS / COLSORT_NT;  // thread i owns the bins COL_BINS-1-PER*i .. COL_BINS-PER-PER*i
   int c[PER], sum = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(256) void psa_bwd_colsort_kernel(const int32_t* cos
   }
   part[tid] = sum;
   __syncthreads();
-  for (int d = 1; d < 256; d <<= 1) {
+  for (int d = 1; d < COLSORT_NT; d <<= 1) {
     const int add = tid >= d ? part[tid - d] : 0;
     __syncthreads();
     part[tid] += add;
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(256) void psa_bwd_colsort_kernel(const int32_t* cos
     run += c[j];
   }
   __syncthreads();
-  for (int i = tid; i < total; i += 256) order[atomicAdd(&hist[cost[i]], 1)] = i;
+  for (int i = tid; i < total; i += COLSORT_NT) order[atomicAdd(&hist[cost[i]], 1)] = i;
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -815,7 +816,7 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       order = cost + n_wg;
       hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, spb, cost);
       if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
-      hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(256), 0, st, cost, (int)n_wg, order);
+      hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(COLSORT_NT), 0, st, cost, (int)n_wg, order);
       if (int e = psa_check_launch("psa_bwd (column order)")) return e;
     }
     auto launch = [&](auto kern) -> int {
