@@ -208,7 +208,10 @@ __global__ __launch_bounds__(X_WAVES * 64, 1) void psa_xattn_gemm_kernel(XParams
 }
 
 // one workgroup per (b, h, q-block): 256 threads; thread t handles key blocks t, t+256, ...
-__global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p) {
+// cached != 0: the (maximum, sum) pairs of the workgroup's rows are read from the workspace once into dynamic LDS
+// ([key block][row], NB * rb pairs) and the three passes below run on that copy instead of on memory.
+__global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p, int cached) {
+  extern __shared__ __align__(16) unsigned char s_cache[];
   __shared__ float s_M[32], s_inv[32];
   __shared__ float s_big[256];
   const int I = blockIdx.x, bh = blockIdx.y;
@@ -216,6 +219,22 @@ __global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p) {
   const int rb = 1 << p.rb_log2;
   const int m0 = I * rb;
   const float* ws = p.ws + (int64_t)bh * p.NB * p.Mr * 2;
+  int64_t row_stride = p.Mr;  // pairs between consecutive key blocks of one row
+  int m_sub = 0;
+  if (cached) {
+    // a key block's rb pairs of this q-block are contiguous in the workspace: rb * 8 bytes per key block
+    f32x2* c = (f32x2*)s_cache;
+    const int jlim = p.causal ? (((m0 + rb - 1 + p.off) >> p.rb_log2) + 1) : p.NB;  // key blocks any row of the q-block sees
+    const int jn = jlim < p.NB ? jlim : p.NB;
+    for (int u = tid; u < jn * rb; u += 256) {
+      const int J = u >> p.rb_log2, rr = u & (rb - 1);
+      c[u] = *(const f32x2*)(ws + ((int64_t)J * p.Mr + m0 + rr) * 2);
+    }
+    __syncthreads();
+    ws = (const float*)s_cache;
+    row_stride = rb;
+    m_sub = m0;  // the copy starts at row m0: index (J * rb + (m - m0)) (never form a pointer below the array)
+  }
   // pass 1: row max and denominator.  Thread (r = tid % rb, jl = tid / rb) strides over the key blocks
   // visible to row r (J <= (m + off) / rb under causality); partials are combined in a fixed order.
   const int r = tid & (rb - 1), jl = tid >> p.rb_log2, nj = 256 >> p.rb_log2;
@@ -223,7 +242,7 @@ __global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p) {
   const int jmax = p.causal ? ((m + p.off) >> p.rb_log2) + 1 : p.NB;
   const int jend = jmax < p.NB ? jmax : p.NB;
   float M = -INFINITY;
-  for (int J = jl; J < jend; J += nj) M = fmaxf(M, ws[((int64_t)J * p.Mr + m) * 2]);
+  for (int J = jl; J < jend; J += nj) M = fmaxf(M, ws[((int64_t)J * row_stride + (m - m_sub)) * 2]);
   s_big[jl * rb + r] = M;
   __syncthreads();
   if (tid < rb) {
@@ -235,7 +254,7 @@ __global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p) {
   const float Mref = s_M[r] == -INFINITY ? 0.f : s_M[r];
   float l = 0.f;
   for (int J = jl; J < jend; J += nj) {
-    const f32x2 pr = *(const f32x2*)(ws + ((int64_t)J * p.Mr + m) * 2);
+    const f32x2 pr = *(const f32x2*)(ws + ((int64_t)J * row_stride + (m - m_sub)) * 2);
     l += pr[1] * fast_exp2(pr[0] - Mref);  // pr = (-inf, 0) for fully masked pairs: 0 * exp2(-inf) = 0
   }
   __syncthreads();
@@ -256,7 +275,7 @@ __global__ __launch_bounds__(256) void psa_xattn_reduce_kernel(XParams p) {
       const int mm = m0 + rr;
       const int jm = p.causal ? ((mm + p.off) >> p.rb_log2) + 1 : p.NB;
       if (J < jm) {
-        const f32x2 pr = *(const f32x2*)(ws + ((int64_t)J * p.Mr + mm) * 2);
+        const f32x2 pr = *(const f32x2*)(ws + ((int64_t)J * row_stride + (mm - m_sub)) * 2);
         const float Mx = s_M[rr] == -INFINITY ? 0.f : s_M[rr];
         e += pr[1] * fast_exp2(pr[0] - Mx) * s_inv[rr];
       }
@@ -341,6 +360,9 @@ extern "C" int psa_estimate_xattn(psa_tensor4 q, psa_tensor4 k, float* est, void
   PSA_REQUIRE(rc == PSA_OK, rc, "psa_estimate_xattn: cannot reserve LDS");
   rc = psa_check_launch("psa_estimate_xattn (contraction)");
   if (rc != PSA_OK) return rc;
-  hipLaunchKernelGGL(psa_xattn_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * Hq)), dim3(256), 0, st, p);
+  // the pairs of one q-block: NB * rb * 8 bytes; cached in LDS when that leaves room for several workgroups per CU
+  const size_t cache_bytes = (size_t)p.NB * ((size_t)1 << p.rb_log2) * 8;
+  const int cached = cache_bytes <= 48 * 1024 ? 1 : 0;
+  hipLaunchKernelGGL(psa_xattn_reduce_kernel, dim3((unsigned)p.out_rows, (unsigned)(B * Hq)), dim3(256), cached ? cache_bytes : 0, st, p, cached);
   return psa_check_launch("psa_estimate_xattn (reduction)");
 }
