@@ -34,7 +34,7 @@ extern "C" int psa_level_map(const float* scores, void* map_out, int map_elem_by
     hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map: cannot reserve %zu bytes of LDS", shmem);
   }
-  int nt = Nk <= 64 ? 64 : (Nk <= 128 ? 128 : 256);
+  const int nt = Nk >= 256 ? 256 : ((Nk + 63) / 64) * 64;  // one thread per score up to 256: idle waves only take up slots
   hipLaunchKernelGGL(psa_level_map_kernel, dim3((unsigned)rows), dim3(nt), shmem, (hipStream_t)stream, p);
   return psa_check_launch("psa_level_map");
 }
@@ -129,7 +129,7 @@ extern "C" int psa_level_map_qwen(const float* scores, void* map_out, int map_el
     hipError_t e = hipFuncSetAttribute((const void*)psa_level_map_qwen_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     PSA_REQUIRE(e == hipSuccess, PSA_ERR_LAUNCH, "psa_level_map_qwen: cannot reserve %zu bytes of LDS", shmem);
   }
-  const int nt = S <= 64 ? 64 : (S <= 128 ? 128 : 256);
+  const int nt = S >= 256 ? 256 : ((S + 63) / 64) * 64;
   hipLaunchKernelGGL(psa_level_map_qwen_kernel, dim3((unsigned)(bh * S)), dim3(nt), shmem, (hipStream_t)stream, p);
   return psa_check_launch("psa_level_map_qwen");
 }
