@@ -27,11 +27,19 @@ and no golden vectors of its own):
                          pooling, single retained block, causal all-1)
   psa_backward_dense     torch.autograd through psa_attention_dense (fp64) and
                          finite differences
-  level_map_qwen         hand-worked rows; golden vectors from the reference's
-                         pure-torch function are not taken -> parity unpinned
-                         beyond the hand-worked rows
-  estimate_xattn         brute force on tiny inputs; parity unpinned otherwise
-  k_similarity           closed form (mean cosine similarity)
+  level_map_qwen         rows worked by hand from the source (topk and energybound, causal on / off,
+                         trailing text rows and columns, later level overwrites, lower bound
+                         max(lo, previous hi), all-zero row) and an independent row-by-row
+                         restatement built from the library calls the reference uses (torch.sort,
+                         cumsum, sum, tensor-vs-scalar arithmetic) on tie-free rows
+  estimate_xattn         brute-force loops in float64: zero-padded tails (L % chunk != 0, padded
+                         keys at logit 0, padded query rows 0), stride 8, causal and not, grouped
+                         heads, Lk > Lq, plus a closed-form case
+  k_similarity           brute-force loops over the explicit token pairs (0,1), (0,3), (0,7) on
+                         random keys with ragged tails, and the library's cosine similarity on
+                         the slices ::2 / 1::2, 0::4 / 3::4, 0::8 / 7::8 of the reference's
+                         pure-torch fall-back
+(the last three: tests/test_oracle_qwen_xattn_ksim.py)
 """
 
 from __future__ import annotations
