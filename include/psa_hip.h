@@ -212,6 +212,20 @@ int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, con
  * (src/psa_triton/kernels/psa_kernel.py:398-431). */
 int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m);
 
+/* psa_fwd without a workspace argument and without any allocation: the row-ordering scratch is a fixed array inside
+ * the library (one copy per GPU, about 0.5 MiB, held until the process ends).  This entry point has no counterpart in
+ * the reference; it exists for callers that cannot allocate device memory around the call - code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It calls no hipMalloc / hipFree or other allocating
+ * routine.  Same arguments, kernels and results (bit for bit) as psa_fwd with a workspace.  Limit: at most
+ * psa_fwd_noalloc_max_rows() = 65536 rows of the level map, rows = B * Hq * ceil(L / block_m); larger shapes return
+ * PSA_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * or threads) race on it and must be serialised by the caller; consecutive calls need no clearing in between. */
+int psa_fwd_noalloc(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+                    const void* map, int map_elem_bytes, psa_tensor4 out, float* lse,
+                    int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
+                    int causal, psa_stream_t stream);
+int64_t psa_fwd_noalloc_max_rows(void);
+
 /* Bytes of workspace psa_bwd needs (fp32 dK/dV per pyramid level, delta, lse in log2 units). */
 int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n);
 

@@ -940,9 +940,9 @@ extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
   return 2 * (total + 16 * FWD_MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
 }
 
-extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
-                       const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
-                       int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
+static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+                    const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
+                    int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
   PSA_REQUIRE(q.ptr && k.ptr && v.ptr && out.ptr, PSA_ERR_ARG, "psa_fwd: null pointer");
   PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_fwd: pooled K/V required with a level map");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
@@ -1015,4 +1015,64 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   else rc = launch_fwd<64, 2>(p, Nk, (hipStream_t)stream);
   PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");
   return psa_check_launch("psa_fwd");
+}
+
+extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+                       const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
+                       int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
+  return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal,
+                  workspace, stream);
+}
+
+// ---- the variant that allocates nothing ------------------------------------------------------------------
+// The row-ordering scratch of psa_fwd (cost and issue order of the rows) lives in a file-scope device array
+// instead of a caller-provided workspace.  Every GPU holds its own copy of the array at its own address; the
+// address is looked up once per device, with that device current, and only that pointer is ever handed to
+// kernels (the array's name is a host-side stand-in, not a device address).
+#include <mutex>
+
+namespace {
+constexpr int64_t FWD_NOALLOC_MAX_ROWS = 1 << 16;  // B * Hq * ceil(L / block_m)
+constexpr size_t FWD_NOALLOC_BYTES = 2 * (size_t)(FWD_NOALLOC_MAX_ROWS + 16 * FWD_MAX_PHASES) * sizeof(int32_t);
+constexpr int FWD_NOALLOC_MAX_DEVICES = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[FWD_NOALLOC_BYTES];
+static void* g_scratch_ptr[FWD_NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+extern "C" int64_t psa_fwd_noalloc_max_rows(void) { return FWD_NOALLOC_MAX_ROWS; }
+
+extern "C" int psa_fwd_noalloc(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
+                               const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv,
+                               int L, int D, int block_m, int block_n, float sm_scale, int causal, psa_stream_t stream) {
+  PSA_REQUIRE(B > 0 && Hq > 0 && L > 0 && block_m > 0, PSA_ERR_ARG, "psa_fwd_noalloc: B, H, L, block_m must be positive");
+  const int64_t rows = (int64_t)B * Hq * ((L + block_m - 1) / block_m);
+  PSA_REQUIRE(rows <= FWD_NOALLOC_MAX_ROWS, PSA_ERR_UNSUPPORTED,
+              "psa_fwd_noalloc: %lld rows of the level map (B * Hq * ceil(L / block_m)) exceed the built-in scratch of %lld rows; "
+              "use psa_fwd with a workspace", (long long)rows, (long long)FWD_NOALLOC_MAX_ROWS);
+  PSA_REQUIRE(psa_fwd_workspace_bytes(B, Hq, L, block_m) <= (int64_t)FWD_NOALLOC_BYTES, PSA_ERR_UNSUPPORTED,
+              "psa_fwd_noalloc: scratch too small for this shape");
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= FWD_NOALLOC_MAX_DEVICES) {
+    psa_set_error("psa_fwd_noalloc: cannot identify the current device");
+    return PSA_ERR_LAUNCH;
+  }
+  void* ptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || p == nullptr) {
+        psa_set_error("psa_fwd_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        return PSA_ERR_LAUNCH;
+      }
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  // every entry of the scratch that a launch reads is written earlier in the same call (row costs, then the issue
+  // order incl. its padding), so nothing has to be cleared between calls
+  return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal, ptr,
+                  stream);
 }

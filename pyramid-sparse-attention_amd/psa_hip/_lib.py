@@ -71,6 +71,12 @@ SIGNATURES = {
          c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     ),
     "psa_fwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int]),
+    "psa_fwd_noalloc": (
+        c_int,
+        [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,
+         c_int, c_int, c_int, c_float, c_int, c_void_p],
+    ),
+    "psa_fwd_noalloc_max_rows": (c_int64, []),
     "psa_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "psa_bwd": (
         c_int,
