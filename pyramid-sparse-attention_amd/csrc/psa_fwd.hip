@@ -39,12 +39,6 @@ namespace {
 #ifndef PSA_FWD_ONE_GROUP
 #define PSA_FWD_ONE_GROUP 0
 #endif
-#ifndef PSA_FWD_LATE_WAIT
-#define PSA_FWD_LATE_WAIT 0
-#endif
-#ifndef PSA_FWD_PRESCALE
-#define PSA_FWD_PRESCALE 0
-#endif
 constexpr int TK = 64;              // pooled keys per tile
 constexpr float LAZY_THRESHOLD = 8.f;  // log2 units the running max may lag behind
 
@@ -418,13 +412,6 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
-#if PSA_FWD_PRESCALE
-    // Q carries the softmax scale (in log2 units) from here on: the logits leave the MFMAs ready for exp2
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) qf[kk][e] = (bf16_t)((float)qf[kk][e] * P_scale_log2);
-#endif
   }
   // both groups run the builder's barriers together
   const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2, P_L,
@@ -496,41 +483,6 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   constexpr int HEAD_PIECES = 12;
   float hx0, hx1, h_cand, h_new;  // state between the pieces
   float alpha = 1.0f, nb = 0.f;
-#if PSA_FWD_PRESCALE
-  // The accumulators of S^T start at (bias - reference maximum), so the MFMAs deliver logits relative to the reference
-  // as it stood BEFORE this tile.  The pieces find the tile's maximum hx0 (relative); the reference is raised only when
-  // the tile exceeds it by more than the threshold (or no key was seen yet), and only then the 32 logits are shifted.
-  float m_base = 0.f, h_delta = 0.f;
-  auto head_piece = [&](int i, f32x16 (&s_cur)[2], bool real) __attribute__((always_inline)) {
-    if (i == 0) {
-      hx0 = s_cur[0][0];
-      hx1 = s_cur[1][0];
-    }
-    if (i < 7) {
-      hx0 = max3f(hx0, s_cur[0][1 + 2 * i], s_cur[0][2 + 2 * i]);
-      hx1 = max3f(hx1, s_cur[1][1 + 2 * i], s_cur[1][2 + 2 * i]);
-    } else if (i == 7) {
-      hx0 = max3f(hx0, s_cur[0][15], fmaxf(hx1, s_cur[1][15]));
-    } else if (i == 8) {
-      hx0 = half_wave_max(hx0);
-    } else if (i == 9) {
-      const bool up = (hx0 > LAZY_THRESHOLD) || (m_run == -INFINITY);
-      h_new = up ? m_base + hx0 : m_run;
-    } else if (i == 10) {
-      const float m_use = h_new == -INFINITY ? 0.f : h_new;  // rows that still see no key
-      alpha = real ? fast_exp2(m_run - m_use) : 1.0f;
-      h_delta = real ? m_base - m_use : 0.f;
-      m_run = real ? h_new : m_run;
-    } else if (i == 11) {
-      if (__any(h_delta != 0.f)) {
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) s_cur[c][e] += h_delta;
-      }
-    }
-  };
-#else
   auto head_piece = [&](int i, const f32x16 (&s_cur)[2], bool real) __attribute__((always_inline)) {
     if (i == 0) {
       hx0 = s_cur[0][0];
@@ -556,19 +508,13 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       m_run = real ? h_new : m_run;
     }
   };
-#endif
   // probabilities of 4 logits: exp2, round to bf16 for P^T; the row sum adds the unrounded values with plain adds
   // (a dot-product instruction would queue behind the other group's MFMAs)
   auto prob4 = [&](const f32x16& sc, int i, float nb_, uint32_t* pk2, float& lsum) __attribute__((always_inline)) {
 #pragma unroll
     for (int e = 0; e < 4; e += 2) {
-#if PSA_FWD_PRESCALE
-      const float p0 = fast_exp2(sc[i + e]);
-      const float p1 = fast_exp2(sc[i + e + 1]);
-#else
       const float p0 = fast_exp2(__builtin_fmaf(sc[i + e], P_scale_log2, nb_));
       const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb_));
-#endif
       pk2[e >> 1] = pack_bf16x2(p0, p1);
       lsum += p0 + p1;
     }
@@ -606,7 +552,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   // latency: all 2*KK K operands are requested up front, and the V^T operands follow into the registers that
   // the QK steps release (two PV steps per k-step), so that the MFMAs stream.  hook(st) runs after PV step st.
   static_assert(4 * DB == 2 * KK, "two PV steps per QK k-step");
-  auto matrix_work = [&](auto kb_c, f32x16 (&s2)[2], const uint32_t (&pk2)[2][8], float a_prev, float c_init, auto mid, auto hook) __attribute__((always_inline)) {
+  auto matrix_work = [&](auto kb_c, f32x16 (&s2)[2], const uint32_t (&pk2)[2][8], float a_prev, auto mid, auto hook) __attribute__((always_inline)) {
     constexpr int KB = decltype(kb_c)::value;
     constexpr int STEPS = 4 * DB;
     PSA_LDS(unsigned char) Ks = (PSA_LDS(unsigned char))(smem_all) + KB * F_TILE;
@@ -624,7 +570,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s2[c][i] = c_init;
+      for (int i = 0; i < 16; ++i) s2[c][i] = 0.f;
     u32x2 vlo[STEPS], vhi[STEPS];
     auto vread = [&](int st) __attribute__((always_inline)) {
       const int cg = st / DB, db = st % DB;
@@ -716,14 +662,8 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     if (T > 0 && t <= T) {
       const bool real = t < T;
       d_cur = real ? d_next : 0u;
-#if PSA_FWD_PRESCALE
-      m_base = m_run == -INFINITY ? 0.f : m_run;
-      const float c_init = (float)(d_cur & 3) - m_base;
-#else
-      const float c_init = 0.f;
-#endif
       matrix_work(
-          cur_c, s, pk, alpha, c_init,
+          cur_c, s, pk, alpha,
           [&]() __attribute__((always_inline)) {
             if (d_cur & 4) mask_tile(t, s);
           },
@@ -741,9 +681,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       const int tn = t + 2 < T ? t + 2 : T_last;
       const u32x2 dd2 = tdesc[tn];
       const uint32_t dn = tdesc[t + 1 < T ? t + 1 : T_last][0];
-#if !PSA_FWD_LATE_WAIT
       __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1), V(t) of this wave have landed (visible to the group after the next barrier)
-#endif
       float lsum = 0.f;
       int n_lv = 0, n_sbs = 0, n_g = 0, n_lim = 0;
       uint16_t n_id = 0;
@@ -779,11 +717,6 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       }
       ts = ts2;
       l_run = l_run * alpha + lsum;
-#if PSA_FWD_LATE_WAIT
-      // K(t+1), V(t) (the 8 copies of the previous vector phase) have landed; the 8 issued above may still be in flight.
-      // The next matrix phase reads them after the barrier that follows.
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-#endif
     }
   };
   if (grp == 1) PP_BARRIER();
