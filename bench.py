@@ -27,27 +27,57 @@ WORKLOADS = {
     # BASELINE.json configs[1]: Wan2.1-1.3B 480p self-attention layer
     "c2": dict(name="wan2.1-1.3b-480p B1 H12 N32760 D128 bf16 blk128 thresholdbound ~90% sparsity",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.90),
-    # BASELINE.json configs[0] (small; run in bf16 on the GPU)
+    # BASELINE.json configs[0] (small; the configuration names fp32 - the kernels compute on bf16 operands with fp32
+    # accumulation, fp32 inputs are rounded to bf16 on entry, and the JSON line says so in `dtype`)
     "c1": dict(name="small B1 H2 N4096 D64 blk64 thresholdbound ~80% sparsity",
-               B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80),
+               B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80,
+               dtype="bf16 (the configuration names fp32: inputs are rounded to bf16 on entry)"),
 }
 WORKLOADS.update({
     # BASELINE.json configs[2]: CogVideoX-5B joint text + video attention (text blocks last, always level 1)
-    "c3": dict(name="cogvideox-5b B2 H48 N17776 (17550 video + 226 text) D64 bf16 blk128 thresholdbound ~85% sparsity",
-               B=2, H=48, grid=(13, 30, 45), D=64, bm=128, bn=128, tn=32, sparsity=0.85, text=226),
+    # (top-k with the ratios of the reference's CogVideo_5b / psa_4steps preset: density 0.15625 before the text columns)
+    "c3": dict(name="cogvideox-5b B2 H48 N17776 (17550 video + 226 text) D64 bf16 blk128 topk psa_4steps ratios ~84% sparsity",
+               B=2, H=48, grid=(13, 30, 45), D=64, bm=128, bn=128, tn=32, sparsity=0.84, text=226, mode="topk",
+               ratios={1: (0.0, 0.05), 2: (0.05, 0.15), 4: (0.15, 0.25), 8: (0.25, 0.5), 0: (0.5, 1.0)}),
     # BASELINE.json configs[3]: training step = forward with lse + backward (dQ, dK, dV)
     "c4": dict(name="training step B1 H12 N32760 D128 bf16 blk128 thresholdbound ~85% sparsity, dO ~ N(0, 0.02)",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.85, kind="train"),
     # BASELINE.json configs[4]: causal GQA prefill at the Qwen2.5-VL-7B decoder shape
     "c5": dict(name="qwen2.5-vl-7b causal prefill B1 Hq28 Hkv4 N32768 (1024 text + 16x44x44 vision) D128 bf16 blk128 "
-                    "energybound ~80% sparsity over the lower triangle",
-               B=1, H=28, Hkv=4, grid=(16, 44, 44), D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal"),
+                    "xattn estimate stride 8, energybound ~80% sparsity over the lower triangle",
+               B=1, H=28, Hkv=4, grid=(16, 44, 44), D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal", stride=8),
 })
 WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
 
 
-# psa_fwd_pp_kernel<128, 4> at workload c2: (850380.5 * 2.000 + 98280.0) KiB per dispatch
-FWD_TRAFFIC_BYTES = {"c2": 1.842e9}
+def fwd_traffic_bytes(workload):
+    """HBM-side bytes per launch of the forward kernel from the committed rocprofv3 counter summary
+    (profiles/psa_layer_c2_kernel_stats.txt, line `roofline.traffic <workload> <kernel> <bytes>`), or None."""
+    path = os.path.join(ROOT, "profiles", "psa_layer_c2_kernel_stats.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 4 and f[0] == "roofline.traffic" and f[1] == workload:
+                return float(f[3])
+    except OSError:
+        pass
+    return None
+
+
+def probe_lib():
+    """bench_probe/libpsa_probe.so (synthetic MFMA / attention-shaped loops; not part of the product library), or None."""
+    import ctypes as ct
+
+    path = os.path.join(PKG, "bench_probe", "libpsa_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ct.CDLL(path)
+    lib.psa_probe_mfma.restype = ct.c_int
+    lib.psa_probe_mfma.argtypes = [ct.c_int, ct.c_int, ct.c_int, ct.c_void_p, ct.c_void_p, ct.POINTER(ct.c_double), ct.c_void_p]
+    lib.psa_probe_attention.restype = ct.c_int
+    lib.psa_probe_attention.argtypes = [ct.c_int, ct.c_int, ct.c_int, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.POINTER(ct.c_double),
+                                        ct.c_void_p]
+    return lib
 
 
 def scaled_ratios(tau):
@@ -83,7 +113,7 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
     if causal:
         # antidiagonal estimate -> causal level map (energy bound scaled to the sparsity target) -> causal GQA forward
         base = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
-        est = ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True)
+        est = ops.estimate_xattn(q, k, block_size=bm, stride=w.get("stride", 8), causal=True)
         lo, hi = 0.05, 1.25
         for _ in range(16):
             tau = 0.5 * (lo + hi)
@@ -93,11 +123,11 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
             lo, hi = (tau, hi) if 1 - dens > w["sparsity"] else (lo, tau)
 
         def step():
-            e = ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True)
+            e = ops.estimate_xattn(q, k, block_size=bm, stride=w.get("stride", 8), causal=True)
             m = ops.level_map_qwen(e, ratios, text, "energybound", block_size=bm, causal=True, map_dtype=torch.int8)
             return ops.sparse_attention_fwd(q, k, v, m, bm, bn, causal=True)
 
-        stages["estimate_xattn"], _ = time_gpu(lambda: ops.estimate_xattn(q, k, block_size=bm, stride=16, causal=True), it)
+        stages["estimate_xattn"], _ = time_gpu(lambda: ops.estimate_xattn(q, k, block_size=bm, stride=w.get("stride", 8), causal=True), it)
         stages["level_map"], _ = time_gpu(lambda: ops.level_map_qwen(est, ratios, text, "energybound", block_size=bm, causal=True,
                                                                     map_dtype=torch.int8), it)
         kp, vp = ops.pool_kv(k, v, bn)
@@ -163,8 +193,9 @@ def run_probe(torch, dev):
     """The synthetic attention-shaped loop of psa_probe_attention, 2 workgroups per CU, about 40-60 ms per variant."""
     import ctypes as ct
 
-    from psa_hip._lib import lib
-
+    lib = probe_lib()
+    if lib is None:
+        raise SystemExit("bench.py --probe needs bench_probe/libpsa_probe.so (python pyramid-sparse-attention_amd/build_ext.py)")
     wgs = torch.cuda.get_device_properties(dev).multi_processor_count * 2
     iters = 25000
     sink = torch.zeros(256, dtype=torch.float32, device=dev)
@@ -242,24 +273,28 @@ def main():
     off_q = sample_offsets(B, H, bm, km, args.seed + 10, device=dev)
     off_k = sample_offsets(B, H, bn, kn, args.seed + 11, device=dev)
 
-    # ---- calibrate tau so that sparsity ~= target (bisection on the level map, untimed) ----
-    scores = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
-    lo, hi = 0.05, 1.25
-    for _ in range(18):
-        tau = 0.5 * (lo + hi)
-        m = ops.level_map(scores, scaled_ratios(tau), text, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
-        dens = float(ops.density(m)[-1])
-        if 1 - dens > w["sparsity"]:
-            lo = tau
-        else:
-            hi = tau
-    ratios = scaled_ratios(tau)
+    mode = w.get("mode", "thresholdbound")
+    if "ratios" in w:
+        ratios, tau = w["ratios"], float("nan")  # a preset of the reference, used as it is
+    else:
+        # ---- calibrate tau so that sparsity ~= target (bisection on the level map, untimed) ----
+        scores = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
+        lo, hi = 0.05, 1.25
+        for _ in range(18):
+            tau = 0.5 * (lo + hi)
+            m = ops.level_map(scores, scaled_ratios(tau), text, mode, blocksize=bn, compute_tile=tn, map_dtype=torch.int8)
+            dens = float(ops.density(m)[-1])
+            if 1 - dens > w["sparsity"]:
+                lo = tau
+            else:
+                hi = tau
+        ratios = scaled_ratios(tau)
 
     state = {}
 
     def layer():
         # estimate -> level map -> pooling -> forward
-        o, mp = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, "thresholdbound", bm, bn, tn, return_map=True, text_length=text)
+        o, mp = ops.psa_layer_fwd(q, k, v, off_q, off_k, ratios, mode, bm, bn, tn, return_map=True, text_length=text)
         state.update(mp=mp, o=o)
         return o
 
@@ -288,7 +323,7 @@ def main():
     it = max(10, min(args.steps, 100))
     t_pool, _ = time_gpu(lambda: ops.pool_kv(k, v, bn), it)
     t_est, _ = time_gpu(lambda: ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn), it)
-    t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
+    t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, text, mode, blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
     out_buf = torch.empty_like(q)
     t_fwd_med, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf), it)
     t_dense = t_sdpa = None
@@ -297,8 +332,9 @@ def main():
         t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
 
     # ---- what the chip sustains on a register-only MFMA loop, measured now (constant and random operands) ----
+    _l = probe_lib()
+
     def mfma_probe(random_operands):
-        from psa_hip._lib import lib as _l
         import ctypes as _ct
         props = torch.cuda.get_device_properties(dev)
         sink = torch.zeros(256, dtype=torch.float32, device=dev)
@@ -319,7 +355,9 @@ def main():
                     "core_clock_ghz": round(float(c[1]) / max(float(c[0]), 1.0) / 10.0, 3)}
         return best
 
-    probe_const, probe_rand, probe_lds = mfma_probe(0), mfma_probe(1), mfma_probe(2)
+    probe_const = probe_rand = probe_lds = None
+    if _l is not None:
+        probe_const, probe_rand, probe_lds = mfma_probe(0), mfma_probe(1), mfma_probe(2)
 
     pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
@@ -333,19 +371,22 @@ def main():
         "frac": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
         # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command (scaled by the
         # readings of --copy-calib's 1 GiB kernel); measured for the default workload only
-        "traffic": FWD_TRAFFIC_BYTES.get(args.workload),
+        "traffic": fwd_traffic_bytes(args.workload),
         "flops_per_launch": exec_flops,
         "avg_launch_ms": round(t_fwd_avg, 4),
         "launch_includes": "the forward kernel and its two row-ordering launches (about 9 us together)",
         # what a register-only loop of independent bf16 MFMAs sustains on this chip right now (psa_probe_mfma, 2 waves
         # per SIMD, 30-45 ms): the clock falls under a dense MFMA stream, further when the operands toggle
-        "mfma_probe_constant_operands": probe_const,
-        "mfma_probe_random_operands": probe_rand,
-        "mfma_probe_random_operands_a_from_lds": probe_lds,
-        "sustained_mfma_tflops_random_operands": probe_rand["tflops"],
-        "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_rand["tflops"], 4),
-        "frac_of_sustained_a_from_lds": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_lds["tflops"], 4),
     }
+    if probe_rand is not None:  # extras, only when the bench-only helper library is built
+        roofline.update({
+            "mfma_probe_constant_operands": probe_const,
+            "mfma_probe_random_operands": probe_rand,
+            "mfma_probe_random_operands_a_from_lds": probe_lds,
+            "sustained_mfma_tflops_random_operands": probe_rand["tflops"],
+            "frac_of_sustained": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_rand["tflops"], 4),
+            "frac_of_sustained_a_from_lds": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / probe_lds["tflops"], 4),
+        })
 
     # ---- CPU baseline: the oracle on the host cores over a bounded sample -------------------
     cpu = None
@@ -361,7 +402,7 @@ def main():
             oqc, okc = off_q[:, heads].cpu(), off_k[:, heads].cpu()
             t0c = time.perf_counter()
             s_c = O.estimate_sampled(qc, kc, bm, bn, oqc, okc)
-            O.level_map(s_c.numpy(), ratios, text, "thresholdbound", blocksize=bn, compute_tile=tn)
+            O.level_map(s_c.numpy(), ratios, text, mode, blocksize=bn, compute_tile=tn)
             t_front = time.perf_counter() - t0c  # pooling is inside blockwalk
             t1c = time.perf_counter()
             O.psa_attention_blockwalk(qc, kc, vc, mc, bm, bn, qblocks=qblocks)
@@ -409,10 +450,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": w.get("dtype", "bf16"),
         "data": "synthetic (seeded smooth 3-D field + noise, logit std ~3)",
         "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
-                   "sparsity": round(1 - density, 4), "tau": round(tau, 4)},
+                   "sparsity": round(1 - density, 4), "mask_mode": mode, "tau": None if tau != tau else round(tau, 4)},
         "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
                       "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4)},
         "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),

@@ -174,24 +174,6 @@ int psa_gather_rows(const psa_tensor4* src, const psa_tensor4* dst, const int* h
 int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk, int causal,
                 float* density_out, psa_stream_t stream);
 
-/* Diagnostic, no counterpart in the reference (bench.py uses it to put the measured MFMA utilisation of the attention
- * kernels next to what the chip sustains): `workgroups` x 4 waves each issue iters x 16 independent bf16 32x32x16 MFMAs
- * from registers (random_operands 0: one constant, 1: pseudo-random values, 2: pseudo-random and the A operand of every
- * MFMA re-read from LDS).  sink: >= 256 floats of device memory
- * (never written in practice), clocks: 2 x int64 of device memory = ticks of the constant 100 MHz counter and of the
- * core clock counter over the loop of the first wave, *flops (host, may be NULL) = floating-point operations issued. */
-int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,
-                   psa_stream_t stream);
-
-/* Diagnostic, no counterpart in the reference (bench.py --probe): an attention-shaped loop on synthetic data - per tile
- * and wave 16 QK MFMAs with one operand from LDS, a minimal softmax over the 32 logits, 16 PV MFMAs; 4 waves per workgroup,
- * free-running.  `features` adds what the real kernels have, one at a time: 1 = a workgroup barrier per tile, 2 = 100 more
- * vector instructions per tile, 4 = 8 global->LDS copies per wave and tile from an L2-resident source, 8 = PV operands
- * through the transposing LDS load, 13 = 1 + 4 + 8, 15 = all of them, 20 = the copies of 4 from a private 64 KiB per wave (fabric-bound).
- * copy_source: workgroups * 256 KiB of device memory; sink, clocks, flops as in psa_probe_mfma. */
-int psa_probe_attention(int workgroups, int iters, int features, const void* copy_source, float* sink, int64_t* clocks,
-                        double* flops, psa_stream_t stream);
-
 /* Sparse attention forward from a level map.  out [B, Hq, L, D] bf16; lse (may be NULL)
  * [B, Hq, L] fp32 = natural-log softmax denominator incl. the +ln(level) bias; map == NULL means
  * dense attention (every pair at level 1; k_pool/v_pool may then be NULL).  K/V have Hkv heads,

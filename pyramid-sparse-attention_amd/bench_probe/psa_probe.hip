@@ -1,3 +1,6 @@
+// Bench-only helper, built into its own small library (bench_probe/libpsa_probe.so); it is not part of libpsa_hip.so
+// and has no entry in the C ABI.  bench.py loads it when present.
+//
 // Diagnostic: the bf16 MFMA rate and the core clock the chip sustains under a pure, register-only MFMA load.
 //
 // The published 2.5 PFLOP/s bf16 peak assumes the boost clock; under a dense MFMA stream the chip lowers its clock
@@ -6,7 +9,11 @@
 // Every wave keeps 4 A and 4 B operands in registers and issues iters * 4 independent 32x32x16 MFMAs on 4
 // accumulators; nothing touches LDS or memory inside the loop (modes 0 and 1), or every MFMA takes its A operand from
 // LDS (mode 2).
-#include "psa_common.h"
+#include "../csrc/psa_common.h"
+
+// (this library stands alone: the error helpers of libpsa_hip.so are replaced by local ones)
+void psa_set_error(const char*, ...) {}
+int psa_check_launch(const char*) { return hipGetLastError() == hipSuccess ? PSA_OK : PSA_ERR_LAUNCH; }
 
 namespace {
 
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(256, 2) void psa_probe_attn_kernel(int iters, const
 }  // namespace
 
 extern "C" int psa_probe_mfma(int workgroups, int iters, int random_operands, float* sink, int64_t* clocks, double* flops,
-                              psa_stream_t stream) {
+                              void* stream) {
   PSA_REQUIRE(workgroups > 0 && iters > 0 && sink && clocks, PSA_ERR_ARG, "psa_probe_mfma: bad arguments");
   hipLaunchKernelGGL(psa_probe_mfma_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream, iters, random_operands, sink,
                      (long long*)clocks);
@@ -195,7 +202,7 @@ extern "C" int psa_probe_mfma(int workgroups, int iters, int random_operands, fl
 }
 
 extern "C" int psa_probe_attention(int workgroups, int iters, int features, const void* copy_source, float* sink, int64_t* clocks,
-                                   double* flops, psa_stream_t stream) {
+                                   double* flops, void* stream) {
   PSA_REQUIRE(workgroups > 0 && iters > 0 && sink && clocks && copy_source, PSA_ERR_ARG, "psa_probe_attention: bad arguments");
   const dim3 g((unsigned)workgroups), b(256);
   hipStream_t st = (hipStream_t)stream;

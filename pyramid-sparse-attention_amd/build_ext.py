@@ -30,7 +30,6 @@ FLAGS = [
 FILE_FLAGS = {
     "psa_fwd.hip": ["-fno-honor-nans"],
     "psa_estimate.hip": ["-fno-honor-nans"],
-    "psa_probe.hip": ["-fno-honor-nans"],  # the synthetic loop is compiled like the forward kernel it models
 }
 
 
@@ -67,7 +66,22 @@ def build(verbose=True, extra_flags=(), out=OUT):
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
     if verbose:
         print("built", out)
+    if out == OUT:
+        build_probe(verbose)
     return out
+
+
+PROBE_SRC = os.path.join(HERE, "bench_probe", "psa_probe.hip")
+PROBE_OUT = os.path.join(HERE, "bench_probe", "libpsa_probe.so")
+
+
+def build_probe(verbose=True):
+    """bench.py's optional helper (synthetic MFMA / attention-shaped loops): a library of its own, outside the C ABI.
+    Compiled like the forward kernel it models."""
+    _run([_hipcc(), *FLAGS, "-fno-honor-nans", "-shared", "-o", PROBE_OUT, PROBE_SRC])
+    if verbose:
+        print("built", PROBE_OUT)
+    return PROBE_OUT
 
 
 if __name__ == "__main__":

@@ -125,7 +125,9 @@ class PyramidAdaptiveBlockSparseAttnTrain(nn.Module):
             self.layer_idx = layer_idx
         self.sparsity_counter += 1
         if self.sparsity_counter <= self.config.warmup_steps:
-            return ops.sparse_attention_fwd(q, k, v, None, 128, 128, causal=self.config.causal_main)
+            # dense and NOT causal, as the reference does during warm-up (scaled_dot_product_attention(q, k, v) without a
+            # mask: qwen2.5-vl-example/src/attention/PSA_casual/PyramidAdaptiveBlockSparseAttn.py:306-308)
+            return ops.sparse_attention_fwd(q, k, v, None, 128, 128, causal=False)
         out, sparsity, per_head = adaptive_block_sparse_attn(q, k, v, self.config, self.sparse_attention_fn,
                                                              compute_stats=self.log_path is not None)
         if self.log_path is not None:

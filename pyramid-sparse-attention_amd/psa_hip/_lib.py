@@ -63,8 +63,6 @@ SIGNATURES = {
     "psa_density": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "psa_gather_rows": (c_int, [POINTER(Tensor4), POINTER(Tensor4), POINTER(c_int), c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
-    "psa_probe_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, POINTER(c_double), c_void_p]),
-    "psa_probe_attention": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, POINTER(c_double), c_void_p]),
     "psa_fwd": (
         c_int,
         [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,

@@ -53,39 +53,30 @@ class GilbertRearranger:
                 and 256 % ((x.shape[-1] * x.element_size()) // 16) == 0 and x.data_ptr() % 16 == 0
                 and all((s * x.element_size()) % 16 == 0 for s in x.stride()[:3]))
 
+    def _check(self, x: torch.Tensor, what: str) -> None:
+        # there is no torch fall-back: tensors the row-gather kernel cannot take are an error, as for every other operator
+        if not (self._native(x) and x.shape[-2] == self.total_elements + self.text_length):
+            raise ValueError(
+                "GilbertRearranger.%s: expected a GPU tensor [B, H, %d, D] with 2- or 4-byte elements, 16-byte aligned rows and "
+                "strides (got shape %s on %s)" % (what, self.total_elements + self.text_length, tuple(x.shape), x.device))
+
     def rearrange_single(self, x: torch.Tensor) -> torch.Tensor:
-        if self._native(x) and x.shape[-2] == self.total_elements + self.text_length:
-            from .. import ops
+        from .. import ops
 
-            return ops.gather_rows((x,), self._combined_index(x.device, True))[0]
-        return self._rearrange_single_torch(x)
-
-    def _rearrange_single_torch(self, x: torch.Tensor) -> torch.Tensor:
-        idx = self._indices(x.device, True)
-        if self.text_length == 0:
-            return x.index_select(-2, idx)
-        text, video = x[..., : self.text_length, :], x[..., self.text_length :, :]
-        return torch.cat((video.index_select(-2, idx), text), dim=-2)
+        self._check(x, "rearrange_single")
+        return ops.gather_rows((x,), self._combined_index(x.device, True))[0]
 
     def rearrange(self, q, k, v) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-        L = self.total_elements + self.text_length
-        if (all(self._native(t) and t.shape[-2] == L for t in (q, k, v)) and q.dtype == k.dtype == v.dtype
-                and q.shape[0] == k.shape[0] == v.shape[0] and q.shape[-1] == k.shape[-1] == v.shape[-1]):
-            from .. import ops
+        from .. import ops
 
+        for t in (q, k, v):
+            self._check(t, "rearrange")
+        if q.dtype == k.dtype == v.dtype and q.shape[0] == k.shape[0] == v.shape[0] and q.shape[-1] == k.shape[-1] == v.shape[-1]:
             return ops.gather_rows((q, k, v), self._combined_index(q.device, True))  # one launch for the three
         return self.rearrange_single(q), self.rearrange_single(k), self.rearrange_single(v)
 
     def reversed_rearrange(self, out: torch.Tensor) -> torch.Tensor:
-        if self._native(out) and out.shape[-2] == self.total_elements + self.text_length:
-            from .. import ops
+        from .. import ops
 
-            return ops.gather_rows((out,), self._combined_index(out.device, False))[0]
-        return self._reversed_rearrange_torch(out)
-
-    def _reversed_rearrange_torch(self, out: torch.Tensor) -> torch.Tensor:
-        idx = self._indices(out.device, False)
-        if self.text_length == 0:
-            return out.index_select(-2, idx)
-        video, text = out[..., : -self.text_length, :], out[..., -self.text_length :, :]
-        return torch.cat((text, video.index_select(-2, idx)), dim=-2)
+        self._check(out, "reversed_rearrange")
+        return ops.gather_rows((out,), self._combined_index(out.device, False))[0]

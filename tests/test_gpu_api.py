@@ -175,54 +175,3 @@ def test_layer_function_equals_the_stages_in_sequence():
         torch.cuda.synchronize()
         assert torch.equal(m2, mp)
         assert torch.equal(out, ref)
-
-
-def test_mfma_probe_runs_and_reports_clocks():
-    """The diagnostic behind bench.py's `frac_of_sustained`: finishes, counts its flops, reads both clocks."""
-    import ctypes
-
-    from psa_hip._lib import lib
-
-    sink = torch.zeros(256, dtype=torch.float32, device=dev())
-    clocks = torch.zeros(2, dtype=torch.int64, device=dev())
-    flops = ctypes.c_double(0.0)
-    for rnd_ops in (0, 1):
-        rc = lib.psa_probe_mfma(64, 500, rnd_ops, ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(clocks.data_ptr()), ctypes.byref(flops),
-                                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-        assert rc == 0
-        torch.cuda.synchronize()
-        c = clocks.cpu()
-        assert flops.value == 64 * 4 * 500 * 16 * 2.0 * 32 * 32 * 16
-        assert int(c[0]) > 0 and 0.5 < float(c[1]) / float(c[0]) / 10.0 < 3.5  # core clock in GHz
-        assert float(sink.abs().sum()) == 0.0
-    assert lib.psa_probe_mfma(0, 500, 0, ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(clocks.data_ptr()), None, None) != 0
-
-
-@pytest.mark.parametrize("features", [0, 1, 2, 4, 8, 13, 15, 20])
-def test_attention_probe_variants_run(features):
-    """bench.py --probe: every variant of the synthetic attention-shaped loop launches, finishes and counts its flops."""
-    import ctypes
-
-    from psa_hip._lib import lib
-
-    wgs, iters = 16, 50
-    sink = torch.zeros(256, dtype=torch.float32, device=dev())
-    clocks = torch.zeros(2, dtype=torch.int64, device=dev())
-    src = torch.zeros(wgs * 256 * 1024, dtype=torch.uint8, device=dev())
-    flops = ctypes.c_double(0.0)
-    rc = lib.psa_probe_attention(wgs, iters, features, ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
-                                 ctypes.c_void_p(clocks.data_ptr()), ctypes.byref(flops), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    assert rc == 0
-    torch.cuda.synchronize()
-    assert flops.value == wgs * 4 * iters * 32 * 2.0 * 32 * 32 * 16
-    assert int(clocks[0]) > 0 and int(clocks[1]) > 0 and float(sink.abs().sum()) == 0.0
-
-
-def test_attention_probe_rejects_unknown_features():
-    import ctypes
-
-    from psa_hip._lib import lib
-
-    buf = torch.zeros(1 << 20, dtype=torch.uint8, device=dev())
-    p = ctypes.c_void_p(buf.data_ptr())
-    assert lib.psa_probe_attention(1, 10, 3, p, p, p, None, None) != 0

@@ -74,10 +74,11 @@ def test_causal_module_end_to_end_gqa():
     ref, _ = O.psa_attention_blockwalk(q, k, v, ref_map, 128, 128, causal=True)
     mx, mean = attn_errors(out, ref)
     assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
-    # warm-up = dense causal attention
+    # warm-up = dense attention WITHOUT a mask, as in the reference (scaled_dot_product_attention(q, k, v);
+    # qwen2.5-vl-example/src/attention/PSA_casual/PyramidAdaptiveBlockSparseAttn.py:306-308)
     warm = PyramidAdaptiveBlockSparseAttnTrain(AttentionConfig(warmup_steps=1))
     o2 = warm(qd, kd, vd)
-    refc = F.scaled_dot_product_attention(q.float(), k.float().repeat_interleave(2, 1), v.float().repeat_interleave(2, 1), is_causal=True)
+    refc = F.scaled_dot_product_attention(q.float(), k.float().repeat_interleave(2, 1), v.float().repeat_interleave(2, 1))
     mx, mean = attn_errors(o2, refc)
     assert mx <= MAX_ABS and mean <= MEAN_ABS
     with pytest.raises(ValueError):

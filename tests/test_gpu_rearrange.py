@@ -20,13 +20,28 @@ def test_rearranger_matches_torch_path(dtype, grid, text, D):
     q = torch.randn(2, 4, L, D, generator=g).to(dtype).to(dev())
     k = torch.randn(2, 2, L, D, generator=g).to(dtype).to(dev())   # fewer heads (GQA)
     v = torch.randn(2, 2, L, D, generator=g).to(dtype).to(dev())
+    fwd = r.original_order2gilbert_order_cpu.to(dev())
+    inv = r.gilbert_order2original_order_cpu.to(dev())
+
+    def ref_forward(x):  # the reference's formulation: index_select of the video part, text appended
+        if text == 0:
+            return x.index_select(-2, fwd)
+        return torch.cat((x[..., text:, :].index_select(-2, fwd), x[..., :text, :]), dim=-2)
+
+    def ref_backward(x):
+        if text == 0:
+            return x.index_select(-2, inv)
+        return torch.cat((x[..., -text:, :], x[..., :-text, :].index_select(-2, inv)), dim=-2)
+
     qr, kr, vr = r.rearrange(q, k, v)
     for a, x in ((qr, q), (kr, k), (vr, v)):
-        assert torch.equal(a, r._rearrange_single_torch(x))
+        assert torch.equal(a, ref_forward(x))
         assert torch.equal(r.rearrange_single(x), a)
     back = r.reversed_rearrange(qr)
-    assert torch.equal(back, r._reversed_rearrange_torch(qr))
+    assert torch.equal(back, ref_backward(qr))
     assert torch.equal(back, q)  # the two orders are inverse permutations
+    with pytest.raises(ValueError):
+        r.rearrange_single(q.cpu())  # no torch fall-back
 
 
 def test_gather_rows_strided_views_and_errors():

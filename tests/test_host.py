@@ -146,16 +146,25 @@ def test_gilbert_curve_golden_and_properties():
 
 
 def test_gilbert_rearranger_round_trip_and_text_position():
+    """The index vectors the row-gather kernel is driven with (pure index arithmetic, checked here with torch indexing
+    on the CPU): text tokens move to the end, the two orders are inverse permutations.  The rearranger itself has no
+    CPU path: a CPU tensor is an error."""
     from psa_hip.utils.rearranger import GilbertRearranger
 
     for text in (0, 5):
         r = GilbertRearranger(6, 4, 3, text)
         n = 72 + text
         x = torch.arange(n, dtype=torch.float32).view(1, 1, n, 1).repeat(1, 2, 1, 3)
-        q, k, v = r.rearrange(x, x + 1000, x + 2000)
-        assert q.shape == x.shape
+        fwd, bwd = r._combined_index("cpu", True).long(), r._combined_index("cpu", False).long()
+        q = x.index_select(2, fwd)
         if text:
             assert q[0, 0, -text:, 0].tolist() == list(range(text))  # text moved to the end
         assert sorted(q[0, 0, :, 0].tolist()) == list(range(n))
-        assert torch.equal(r.reversed_rearrange(q), x) and torch.equal(r.reversed_rearrange(v), x + 2000)
-        assert torch.equal(r.rearrange_single(x), q)
+        assert torch.equal(q.index_select(2, bwd), x)
+        # the same as the reference's formulation: index_select of the video part, text appended
+        ref = torch.cat((x[:, :, text:].index_select(2, r.original_order2gilbert_order_cpu), x[:, :, :text]), 2)
+        assert torch.equal(q, ref)
+        with pytest.raises(ValueError):
+            r.rearrange(x, x, x)
+        with pytest.raises(ValueError):
+            r.reversed_rearrange(x)
