@@ -106,44 +106,6 @@ def adaptive_block_sparse_attn(q, k, v, config, sparse_attention_fn, compute_sta
     return out, sparsity, per_head, sim_cap
 
 
-class _DensityLog:
-    """JSONL sparsity log: one line per layer call.  Values are kept as device tensors and only
-    brought to the host when the log is flushed, so logging does not synchronise every layer."""
-
-    def __init__(self, log_dir, config, model_type, layer_num, inference_num):
-        self.dir = os.path.join(log_dir, time.strftime("%Y%m%d_%H%M%S"))
-        os.makedirs(self.dir, exist_ok=True)
-        cfg = {k: (v if not isinstance(v, dict) else {str(a): list(b) for a, b in v.items()}) for k, v in asdict(config).items()}
-        with open(os.path.join(self.dir, "config.json"), "w") as f:
-            json.dump(dict(config=cfg, model_type=model_type, layer_num=layer_num, inference_num=inference_num), f, indent=1)
-        self.pending = []
-        self.closed = False
-
-    def log_sparsity(self, **kw):
-        self.pending.append(kw)
-        if len(self.pending) >= 256:
-            self.flush()
-
-    def flush(self):
-        if not self.pending:
-            return
-        with open(os.path.join(self.dir, "sparsity.jsonl"), "a") as f:
-            for rec in self.pending:
-                sp, ph = rec["sparsity"], rec["per_head_density"]
-                sp = float(sp) if torch.is_tensor(sp) else sp
-                ph = [float(x) for x in ph.cpu()] if torch.is_tensor(ph) else list(ph)
-                line = dict(layer_idx=rec["layer_idx"], sparsity=sp, density=1 - sp, per_head_density=ph,
-                            sequence_length=rec["sequence_length"], batch_size=rec["batch_size"], num_heads=rec["num_heads"],
-                            is_warmup=rec["is_warmup"])
-                f.write(json.dumps(line) + "\n")
-        self.pending = []
-
-    def close(self):
-        if not self.closed:
-            self.flush()
-            self.closed = True
-
-
 class PyramidSparseAttention(nn.Module):
     """One instance is shared by every transformer block: forward(q, k, v, layer_idx)."""
 
@@ -177,7 +139,9 @@ class PyramidSparseAttention(nn.Module):
             raise ValueError(f"Unknown attn_impl: {config.attn_impl}")
         self.logger = None
         if config.enable_logging:
-            self.logger = _DensityLog(config.log_dir, config, model_type, layer_num, inference_num)
+            from .utils.psa_logger import PSALogger
+
+            self.logger = PSALogger(config.log_dir, config, model_type, layer_num, inference_num)
 
     def get_current_time(self):
         """Denoising step index derived from the call counter (Wan runs cond + uncond per step)."""
@@ -192,12 +156,13 @@ class PyramidSparseAttention(nn.Module):
             q_r, k_r, v_r = q, k, v
         is_warmup = self.get_current_time() < self.config.warmup_steps
         compute_stats = self.config.verbose or self.logger is not None
+        sim_cap = None
         if is_warmup:
             out_r = ops.sparse_attention_fwd(q_r, k_r, v_r, None, 128, 128)  # dense attention, same kernel
             sparsity = 0.0
             per_head_density = [1.0] * q_r.shape[1] if compute_stats else []
         else:
-            out_r, sparsity, per_head_density, _ = adaptive_block_sparse_attn(
+            out_r, sparsity, per_head_density, sim_cap = adaptive_block_sparse_attn(
                 q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets
             )
             if compute_stats:
@@ -205,7 +170,8 @@ class PyramidSparseAttention(nn.Module):
         self.sparsity_counter += 1
         if self.logger is not None:
             self.logger.log_sparsity(layer_idx=layer_idx, sparsity=sparsity, per_head_density=per_head_density,
-                                     sequence_length=q.shape[2], batch_size=q.shape[0], num_heads=q.shape[1], is_warmup=is_warmup)
+                                     sequence_length=q.shape[2], batch_size=q.shape[0], num_heads=q.shape[1], sim_mask=sim_cap,
+                                     is_warmup=is_warmup)
         return self.rearranger.reversed_rearrange(out_r) if self.rearranger is not None else out_r
 
     def close_logger(self):

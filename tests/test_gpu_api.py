@@ -142,6 +142,12 @@ def test_pyramid_sparse_attention_warmup_rearrange_and_logging(tmp_path):
     lines = [json.loads(l) for f in logs if f.endswith("sparsity.jsonl") for l in open(f)]
     assert len(lines) == 8 and lines[0]["is_warmup"] and not lines[-1]["is_warmup"]
     assert 0.0 < lines[-1]["sparsity"] < 1.0 and len(lines[-1]["per_head_density"]) == 2
+    # the reference's schema: running step number, time stamp, similarity-cap histogram (this preset uses the cap)
+    assert [l["global_step"] for l in lines] == list(range(1, 9)) and all("timestamp" in l for l in lines)
+    assert lines[-1]["use_sim_mask"] and abs(sum(lines[-1]["sim_mask_stats"].values()) - 1.0) < 1e-5
+    assert sum(lines[0]["sim_mask_stats"].values()) == 0.0  # warm-up calls carry no cap
+    summary = [f for f in logs if f.endswith("summary.txt")]
+    assert len(summary) == 1 and "Warmup Samples (density=1.0): 4" in open(summary[0]).read()
 
 
 def test_pyramid_sparse_attention_text_tokens_cogvideo_preset():

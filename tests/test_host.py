@@ -168,3 +168,33 @@ def test_gilbert_rearranger_round_trip_and_text_position():
             r.rearrange(x, x, x)
         with pytest.raises(ValueError):
             r.reversed_rearrange(x)
+
+
+def test_psa_logger_schema_and_summary(tmp_path):
+    """The sparsity log keeps the reference's files and fields (src/psa_triton/utils/psa_logger.py:179-286, 314-515);
+    values may arrive as tensors and are only read when the queue is flushed."""
+    from psa_hip.pyramid_sparse_attention import AttentionConfig
+    from psa_hip.utils.psa_logger import PSALogger
+
+    cfg = AttentionConfig(enable_logging=False, use_sim_mask=True, attn_impl="old_mask_type")
+    with PSALogger(str(tmp_path), cfg, "wan", layer_num=2, inference_num=3, session_name="s") as lg:
+        cap = torch.tensor([[[1, 2, 2, 8], [4, 4, 1, 1]]])  # 3/8 at 1x, 2/8 at 2x, 2/8 at 4x, 1/8 at 8x
+        lg.log_sparsity(0, 0.0, [1.0, 1.0], 100, 1, 2, sim_mask=None, is_warmup=True)
+        lg.log_sparsity(0, torch.tensor(0.9), torch.tensor([0.05, 0.15]), 100, 1, 2, sim_mask=cap, is_warmup=False)
+        lg.log_sparsity(1, 0.8, [0.2, 0.2], 100, 1, -1, sim_mask=cap, is_warmup=False)
+        assert not os.path.getsize(tmp_path / "s" / "sparsity.jsonl")  # nothing is read or written before the flush
+    lines = [json.loads(l) for l in open(tmp_path / "s" / "sparsity.jsonl")]
+    assert [l["global_step"] for l in lines] == [1, 2, 3]
+    keys = {"global_step", "timestamp", "layer_idx", "sparsity", "density", "per_head_density", "sequence_length", "batch_size",
+            "num_heads", "is_warmup", "use_sim_mask", "sim_mask_stats"}
+    assert all(set(l) == keys for l in lines)
+    assert lines[1]["sparsity"] == 0.9 and lines[1]["density"] == 0.1 and lines[1]["per_head_density"] == [0.05, 0.15]
+    assert lines[1]["sim_mask_stats"] == {"pool_1x_ratio": 0.375, "pool_2x_ratio": 0.25, "pool_4x_ratio": 0.25, "pool_8x_ratio": 0.125}
+    assert lines[0]["is_warmup"] and lines[0]["sim_mask_stats"]["pool_1x_ratio"] == 0.0 and lines[2]["num_heads"] == 2
+    summary = open(tmp_path / "s" / "summary.txt").read()
+    for needle in ("PSA Sparsity Summary - s", "Total Forward Passes: 3", "Per-Layer Statistics:", "Overall Statistics:",
+                   "Non-Warmup Statistics (excluding density=1.0 steps):", "Warmup Samples (density=1.0): 1",
+                   "Sim Mask Statistics (Average Pooling Distribution):", "1x Pooling (no pooling):  37.50%", "Total Sim Mask Samples:   2"):
+        assert needle in summary, needle
+    cfgj = json.load(open(tmp_path / "s" / "config.json"))
+    assert cfgj["model_type"] == "wan" and cfgj["layer_num"] == 2 and cfgj["config"]["attn_impl"] == "old_mask_type"
