@@ -331,6 +331,34 @@ def main():
         t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
         t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
 
+    # ---- token re-ordering: the layer on tokens already in curve order (above), the same layer reading / writing through
+    # the token index (no gather passes), and with explicit gather passes before and after; the inputs of the last two
+    # are the un-gathered q, k, v, so all three compute the same layer and the outputs must agree bit for bit
+    from psa_hip.utils.rearranger import GilbertRearranger
+
+    gd, gh, gw = w["grid"]
+    rr = GilbertRearranger(gw, gh, gd, text)
+    idx = rr.token_index(dev)
+    inv = rr._combined_index(dev, False)
+    q0, k0, v0 = ops.gather_rows((q, k, v), inv)  # q0[idx[i]] = q[i]
+
+    def layer_indexed():
+        return ops.psa_layer_fwd(q0, k0, v0, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text, token_index=idx)
+
+    def layer_gathered():
+        qg, kg, vg = ops.gather_rows((q0, k0, v0), idx)
+        og = ops.psa_layer_fwd(qg, kg, vg, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text)
+        return ops.gather_rows((og,), inv)[0]
+
+    o_ref = layer()
+    reorder_equal = bool(torch.equal(layer_indexed(), layer_gathered())) and bool(torch.equal(ops.gather_rows((layer_indexed(),), idx)[0], o_ref))
+    t_l0, _ = time_gpu(layer, it)
+    t_l1, _ = time_gpu(layer_indexed, it)
+    t_l2, _ = time_gpu(layer_gathered, it)
+    reorder = {"layer_tokens_already_ordered": round(t_l0, 4), "layer_through_token_index": round(t_l1, 4),
+               "layer_with_gather_passes": round(t_l2, 4), "outputs_bit_identical": reorder_equal}
+    del q0, k0, v0
+
     # ---- what the chip sustains on a register-only MFMA loop, measured now (constant and random operands) ----
     _l = probe_lib()
 
@@ -456,6 +484,7 @@ def main():
                    "sparsity": round(1 - density, 4), "mask_mode": mode, "tau": None if tau != tau else round(tau, 4)},
         "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
                       "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4)},
+        "reorder_ms": reorder,
         "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),
         "pct_bf16_peak_fwd_executed": round(100 * exec_flops / (t_fwd_med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
         "pool_gbs": round(pool_bytes / (t_pool * 1e-3) / 1e9, 1),

@@ -168,6 +168,35 @@ int psa_gather_rows(const psa_tensor4* src, const psa_tensor4* dst, const int* h
                     const int32_t* index, int B, int L_dst, int L_src, int D, int elem_bytes,
                     psa_stream_t stream);
 
+/* Token re-ordering folded into the layer's own kernels (no separate gather pass over Q, K, V and the output).
+ * index: int32 [L], a permutation of 0..L-1; position i of the re-ordered sequence is source row index[i].
+ *   psa_pool_kv_indexed          pools the re-ordered K, V (the result psa_pool_kv gives on the gathered tensors, bit for
+ *                                bit) and also writes the re-ordered rows themselves to k_ord, v_ord [B, Hkv, L, D]: the
+ *                                level-1 keys / values the attention kernel reads.
+ *   psa_estimate_sampled_indexed, psa_estimate_sampled_map_indexed
+ *                                the estimator with q read through the index (k is passed already re-ordered: k_ord).
+ *   psa_fwd_indexed              the attention kernel with q read through the index and row i of the result (and of lse)
+ *                                written to row index[i] of out: out comes back in the caller's original token order.
+ * Together they give exactly what gather -> layer -> inverse gather gives.  Other arguments as in the functions they
+ * extend.  Replaces GilbertRearranger.rearrange before and reversed_rearrange after the attention call:
+ *   reference src/psa_triton/utils/rearranger.py:14-132 as used at src/psa_triton/pyramid_sparse_attention.py:326-344,386-400. */
+int psa_pool_kv_indexed(psa_tensor4 k, psa_tensor4 v, const int32_t* index, psa_tensor4 k_ord, psa_tensor4 v_ord,
+                        void* k_pool, void* v_pool, int B, int Hkv, int L, int D, int block_n, psa_stream_t stream);
+int psa_estimate_sampled_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, const int32_t* off_q,
+                                 const int32_t* off_k, float* scores, void* workspace, int B, int Hq, int Hkv, int Lq,
+                                 int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                                 int out_rows, int out_cols, psa_stream_t stream);
+int psa_estimate_sampled_map_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, const int32_t* off_q,
+                                     const int32_t* off_k, float* scores, void* workspace, int B, int Hq, int Hkv, int Lq,
+                                     int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                                     int out_rows, int out_cols, void* map_out, int map_elem_bytes, int mode, int n_items,
+                                     const int32_t* item_level, const double* item_hi, int align_div, int text_blocks,
+                                     double min_full_attn_ratio, psa_stream_t stream);
+int psa_fwd_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
+                    const void* v_pool, const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq,
+                    int Hkv, int L, int D, int block_m, int block_n, float sm_scale, int causal, void* workspace,
+                    psa_stream_t stream);
+
 /* mean(1/level) over the map, skipped blocks counting 0; causal != 0 counts lower-triangle pairs only.
  * density_out: one float per (b, h) row of the [BH] vector, plus the overall mean at index BH.
  * reference src/psa_triton/utils/transfer_attn_to_mask.py:510-544. */

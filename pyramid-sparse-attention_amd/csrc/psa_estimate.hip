@@ -28,6 +28,7 @@ struct EstParams {
   const bf16_t *q, *k;
   int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl;
   const int32_t *off_q, *off_k;
+  const int32_t* q_index;  // optional: the sampled query position i is source row q_index[i] (token re-ordering)
   float* rt;   // workspace: R^T [B*Hq][n_d][Ms_pad]
   float* mrow; // workspace: m [B*Hq][ksplit][Ms_pad]: row maxima over each share of the keys
   int ksplit;  // the key range is cut into ksplit shares (grid z) to even out the load
@@ -107,7 +108,8 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
     const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * keep_m : nullptr;
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
-      const int src = sampled_src(row0 + rs * 32 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
+      int src = sampled_src(row0 + rs * 32 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
+      if (p.q_index != nullptr) src = p.q_index[src];
       const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) qf[rs][kk] = *(const bf16x8*)(qp + kk * 16);
@@ -379,7 +381,8 @@ extern "C" int64_t psa_estimate_workspace_bytes(int B, int Hq, int Lq, int Lk, i
 }
 
 namespace {
-int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores, void* workspace, int B, int Hq,
+int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, const int32_t* q_index, float* scores,
+            void* workspace, int B, int Hq,
             int Hkv, int Lq, int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale, int out_rows,
             int out_cols, LevelMapParams* lp, bool* map_done, psa_stream_t stream) {
   PSA_REQUIRE(q.ptr && k.ptr && (scores || lp) && workspace, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
@@ -400,7 +403,7 @@ int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* o
   p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr;
   p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sl = q.stride_l;
   p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sl = k.stride_l;
-  p.off_q = off_q; p.off_k = off_k; p.scores = scores;
+  p.off_q = off_q; p.off_k = off_k; p.q_index = q_index; p.scores = scores;
   p.Hq = Hq; p.Hkv = Hkv; p.Lq = Lq; p.Lk = Lk; p.bm = block_m; p.bn = block_n;
   p.keep_m_log2 = psa_ilog2(keep_m); p.keep_n_log2 = psa_ilog2(keep_n);
   p.Ms = g.Ms; p.Ns = g.Ns; p.Ms_pad = g.Ms_pad; p.Ns_pad = g.Ns_pad; p.n_d = g.n_d;
@@ -423,15 +426,25 @@ extern "C" int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t*
                                     int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, psa_stream_t stream) {
   PSA_REQUIRE(scores, PSA_ERR_ARG, "psa_estimate_sampled: null pointer");
   bool unused = false;
-  return est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale, out_rows,
-                 out_cols, nullptr, &unused, stream);
+  return est_run(q, k, off_q, off_k, nullptr, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
+                 out_rows, out_cols, nullptr, &unused, stream);
 }
 
-extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
-                                        void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
-                                        int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, void* map_out,
-                                        int map_elem_bytes, int mode, int n_items, const int32_t* item_level, const double* item_hi,
-                                        int align_div, int text_blocks, double min_full_attn_ratio, psa_stream_t stream) {
+extern "C" int psa_estimate_sampled_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, const int32_t* off_q,
+                                            const int32_t* off_k, float* scores, void* workspace, int B, int Hq, int Hkv, int Lq,
+                                            int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                                            int out_rows, int out_cols, psa_stream_t stream) {
+  PSA_REQUIRE(scores && q_index, PSA_ERR_ARG, "psa_estimate_sampled_indexed: null pointer");
+  bool unused = false;
+  return est_run(q, k, off_q, off_k, q_index, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
+                 out_rows, out_cols, nullptr, &unused, stream);
+}
+
+static int est_map_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, const int32_t* q_index, float* scores,
+                       void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
+                       int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, void* map_out,
+                       int map_elem_bytes, int mode, int n_items, const int32_t* item_level, const double* item_hi,
+                       int align_div, int text_blocks, double min_full_attn_ratio, psa_stream_t stream) {
   PSA_REQUIRE(map_out, PSA_ERR_ARG, "psa_estimate_sampled_map: null pointer");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_estimate_sampled_map: map_elem_bytes must be 1 or 4");
   PSA_REQUIRE(out_cols > 0, PSA_ERR_ARG, "psa_estimate_sampled_map: out_cols must be positive");
@@ -440,9 +453,31 @@ extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int3
   if (rc != PSA_OK) return rc;
   lp.map_out = map_out; lp.map_elem = map_elem_bytes;
   bool map_done = false;
-  const int rc2 = est_run(q, k, off_q, off_k, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
-                          out_rows, out_cols, &lp, &map_done, stream);
+  const int rc2 = est_run(q, k, off_q, off_k, q_index, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n,
+                          sm_scale, out_rows, out_cols, &lp, &map_done, stream);
   if (rc2 != PSA_OK || map_done) return rc2;
   return psa_level_map(scores, map_out, map_elem_bytes, nullptr, (int64_t)B * Hq * out_rows, out_cols, mode, n_items, item_level, item_hi,
                        align_div, text_blocks, min_full_attn_ratio, stream);
+}
+
+extern "C" int psa_estimate_sampled_map(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* off_k, float* scores,
+                                        void* workspace, int B, int Hq, int Hkv, int Lq, int Lk, int D, int block_m, int block_n,
+                                        int keep_m, int keep_n, float sm_scale, int out_rows, int out_cols, void* map_out,
+                                        int map_elem_bytes, int mode, int n_items, const int32_t* item_level, const double* item_hi,
+                                        int align_div, int text_blocks, double min_full_attn_ratio, psa_stream_t stream) {
+  return est_map_run(q, k, off_q, off_k, nullptr, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
+                     out_rows, out_cols, map_out, map_elem_bytes, mode, n_items, item_level, item_hi, align_div, text_blocks,
+                     min_full_attn_ratio, stream);
+}
+
+extern "C" int psa_estimate_sampled_map_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, const int32_t* off_q,
+                                                const int32_t* off_k, float* scores, void* workspace, int B, int Hq, int Hkv, int Lq,
+                                                int Lk, int D, int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
+                                                int out_rows, int out_cols, void* map_out, int map_elem_bytes, int mode, int n_items,
+                                                const int32_t* item_level, const double* item_hi, int align_div, int text_blocks,
+                                                double min_full_attn_ratio, psa_stream_t stream) {
+  PSA_REQUIRE(q_index != nullptr, PSA_ERR_ARG, "psa_estimate_sampled_map_indexed: null index");
+  return est_map_run(q, k, off_q, off_k, q_index, scores, workspace, B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, sm_scale,
+                     out_rows, out_cols, map_out, map_elem_bytes, mode, n_items, item_level, item_hi, align_div, text_blocks,
+                     min_full_attn_ratio, stream);
 }

@@ -58,6 +58,7 @@ struct FwdParams {
   int max_tiles;
   int grp_bytes;  // two-group kernel: LDS bytes of one group (tile buffers + schedule)
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
+  const int32_t* q_index;  // optional (token re-ordering): query / output position i lives in row q_index[i] of q, out, lse
 };
 
 constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the blocks of a tile
@@ -115,7 +116,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   const int q_idx = q_row0 + l32;
   bf16x8 qf[KK];
   {
-    const int qr = q_idx < P_L ? q_idx : P_L - 1;
+    int qr = q_idx < P_L ? q_idx : P_L - 1;
+    if (p.q_index != nullptr) qr = p.q_index[qr];
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
@@ -319,7 +321,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   const float inv = 1.0f / l_safe;
   if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
     // natural-log domain: m*ln2 + ln(max(l, 1e-8))
-    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+    p.lse[((int64_t)b * p.Hq + h) * P_L + (p.q_index != nullptr ? p.q_index[q_idx] : q_idx)] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
   }
   __syncthreads();  // everyone is done with the last K/V tile
   unsigned char* Os = smem;
@@ -337,7 +339,10 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   for (int u = tid; u < BM * CH; u += NT) {
     const int r = u / CH, ch = u % CH;
     const int row = I * BM + r;
-    if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+    if (row < P_L) {
+      const int orow = p.q_index != nullptr ? p.q_index[row] : row;
+      *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+    }
   }
 }
 
@@ -408,7 +413,8 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   const int q_idx = q_row0 + l32;
   bf16x8 qf[KK];
   {
-    const int qr = q_idx < P_L ? q_idx : P_L - 1;
+    int qr = q_idx < P_L ? q_idx : P_L - 1;
+    if (p.q_index != nullptr) qr = p.q_index[qr];
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
@@ -737,7 +743,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   const float l_safe = fmaxf(l_tot, 1e-8f);
   const float inv = 1.0f / l_safe;
   if (active && p.lse != nullptr && hh == 0 && q_idx < P_L) {
-    p.lse[((int64_t)b * p.Hq + h) * P_L + q_idx] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+    p.lse[((int64_t)b * p.Hq + h) * P_L + (p.q_index != nullptr ? p.q_index[q_idx] : q_idx)] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // the last (repeated) tile copies land in the buffers that now stage O
   __syncthreads();
@@ -757,7 +763,10 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     for (int u = tid; u < BM * CH; u += NT) {
       const int r = u / CH, ch = u % CH;
       const int row = I * BM + r;
-      if (row < P_L) *(u32x4*)(ob + (int64_t)row * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+      if (row < P_L) {
+        const int orow = p.q_index != nullptr ? p.q_index[row] : row;
+        *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+      }
     }
   }
 }
@@ -875,7 +884,8 @@ extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
 
 static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
                     const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
-                    int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
+                    int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream,
+                    const int32_t* q_index = nullptr) {
   PSA_REQUIRE(q.ptr && k.ptr && v.ptr && out.ptr, PSA_ERR_ARG, "psa_fwd: null pointer");
   PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_fwd: pooled K/V required with a level map");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
@@ -929,6 +939,7 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
                          (int64_t)Nk * block_n < (1 << 24) && k.stride_l * 2 < (1 << 24) && v.stride_l * 2 < (1 << 24);
   if (two_group) p.wg_chunk = (p.wg_chunk + 1) & ~1;  // pairs never straddle two groups of rows
   p.order = nullptr;
+  p.q_index = q_index;
   if (workspace != nullptr && map != nullptr && total > 8 * 32) {
     PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
     int32_t* order = (int32_t*)workspace;
@@ -955,6 +966,15 @@ extern "C" int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
                        int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream) {
   return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal,
                   workspace, stream);
+}
+
+extern "C" int psa_fwd_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
+                               const void* v_pool, const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq,
+                               int Hkv, int L, int D, int block_m, int block_n, float sm_scale, int causal, void* workspace,
+                               psa_stream_t stream) {
+  PSA_REQUIRE(q_index != nullptr, PSA_ERR_ARG, "psa_fwd_indexed: null index");
+  return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal,
+                  workspace, stream, q_index);
 }
 
 // ---- the variant that allocates nothing ------------------------------------------------------------------

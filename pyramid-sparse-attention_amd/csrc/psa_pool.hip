@@ -4,6 +4,10 @@
 // group of D/8 neighbouring lanes reads whole rows; the three levels are reduced in registers and each
 // level is rounded to bf16 before it feeds the next (the reference materialises every level in bf16).
 // Rows past L replicate row L-1 (replicate padding to a multiple of block_n).
+//
+// Indexed form (token re-ordering fused into the pass): position i of the sequence that is pooled is source row
+// index[i]; the re-ordered rows themselves are written out as well (the level-1 keys / values of the attention
+// kernel), so no separate gather pass over K and V is needed.
 #include "psa_common.h"
 
 struct PoolParams {
@@ -12,6 +16,9 @@ struct PoolParams {
   bf16_t* dst[2];
   int H, L, D;
   int64_t npad;
+  const int32_t* index;  // indexed form: source row of every position, else null
+  bf16_t* ord[2];        // indexed form: the re-ordered rows [B, H, L, D] (strides ob / oh / ol)
+  int64_t ob[2], oh[2], ol[2];
 };
 
 __device__ __forceinline__ void unpack8(const u32x4& w, float* f) {
@@ -37,6 +44,7 @@ __device__ __forceinline__ u32x4 mean2(const float* a, const float* b, float* ou
   return r;
 }
 
+template <bool INDEXED>
 __global__ __launch_bounds__(256) void psa_pool_kernel(PoolParams p) {
   const int which = blockIdx.z;
   const int bh = blockIdx.y;
@@ -54,8 +62,12 @@ __global__ __launch_bounds__(256) void psa_pool_kernel(PoolParams p) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     int64_t row = g * 8 + i;
-    row = row < p.L ? row : (int64_t)(p.L - 1);
-    u32x4 w = *(const u32x4*)(src + row * sl);
+    const bool real = row < p.L;
+    row = real ? row : (int64_t)(p.L - 1);
+    const int64_t srow = INDEXED ? (int64_t)p.index[row] : row;
+    u32x4 w = *(const u32x4*)(src + srow * sl);
+    if (INDEXED && real)
+      __builtin_nontemporal_store(w, (u32x4*)(p.ord[which] + b * p.ob[which] + h * p.oh[which] + row * p.ol[which] + c * 8));
     unpack8(w, f[i]);
   }
   float l2[4][8], l4[2][8], l8[8];
@@ -81,8 +93,8 @@ __global__ __launch_bounds__(256) void psa_pool_kernel(PoolParams p) {
   __builtin_nontemporal_store(o8, (u32x4*)(d8 + ((int64_t)bh * (p.npad >> 3) + g) * D + c * 8));
 }
 
-extern "C" int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_pool, int B, int Hkv, int L, int D,
-                           int block_n, psa_stream_t stream) {
+static int pool_run(psa_tensor4 k, psa_tensor4 v, const int32_t* index, const psa_tensor4* k_ord, const psa_tensor4* v_ord,
+                    void* k_pool, void* v_pool, int B, int Hkv, int L, int D, int block_n, psa_stream_t stream) {
   PSA_REQUIRE(k.ptr && v.ptr && k_pool && v_pool, PSA_ERR_ARG, "psa_pool_kv: null pointer");
   PSA_REQUIRE(B > 0 && Hkv > 0 && L > 0, PSA_ERR_ARG, "psa_pool_kv: B, Hkv, L must be positive");
   PSA_REQUIRE(D > 0 && D % 8 == 0 && D <= 256, PSA_ERR_UNSUPPORTED, "psa_pool_kv: D=%d must be a multiple of 8, <= 256", D);
@@ -100,8 +112,35 @@ extern "C" int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_p
   p.dst[1] = (bf16_t*)v_pool;
   p.H = Hkv; p.L = L; p.D = D;
   p.npad = (int64_t)((L + block_n - 1) / block_n) * block_n;
+  p.index = index;
+  p.ord[0] = p.ord[1] = nullptr;
+  p.ob[0] = p.ob[1] = p.oh[0] = p.oh[1] = p.ol[0] = p.ol[1] = 0;
+  if (index != nullptr) {
+    const psa_tensor4* o[2] = {k_ord, v_ord};
+    for (int t = 0; t < 2; ++t) {
+      PSA_REQUIRE(o[t] && o[t]->ptr && ((uintptr_t)o[t]->ptr % 16 == 0) && o[t]->stride_l % 8 == 0 && o[t]->stride_h % 8 == 0 &&
+                      o[t]->stride_b % 8 == 0,
+                  PSA_ERR_ARG, "psa_pool_kv_indexed: the re-ordered outputs must be 16-byte aligned with strides that are multiples of 8");
+      p.ord[t] = (bf16_t*)o[t]->ptr;
+      p.ob[t] = o[t]->stride_b; p.oh[t] = o[t]->stride_h; p.ol[t] = o[t]->stride_l;
+    }
+  }
   int64_t units = (p.npad / 8) * (D / 8);
   dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * Hkv), 2);
-  hipLaunchKernelGGL(psa_pool_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
+  if (index != nullptr)
+    hipLaunchKernelGGL(psa_pool_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL(psa_pool_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
   return psa_check_launch("psa_pool_kv");
+}
+
+extern "C" int psa_pool_kv(psa_tensor4 k, psa_tensor4 v, void* k_pool, void* v_pool, int B, int Hkv, int L, int D,
+                           int block_n, psa_stream_t stream) {
+  return pool_run(k, v, nullptr, nullptr, nullptr, k_pool, v_pool, B, Hkv, L, D, block_n, stream);
+}
+
+extern "C" int psa_pool_kv_indexed(psa_tensor4 k, psa_tensor4 v, const int32_t* index, psa_tensor4 k_ord, psa_tensor4 v_ord,
+                                   void* k_pool, void* v_pool, int B, int Hkv, int L, int D, int block_n, psa_stream_t stream) {
+  PSA_REQUIRE(index != nullptr, PSA_ERR_ARG, "psa_pool_kv_indexed: null index");
+  return pool_run(k, v, index, &k_ord, &v_ord, k_pool, v_pool, B, Hkv, L, D, block_n, stream);
 }

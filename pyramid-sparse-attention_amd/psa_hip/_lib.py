@@ -63,6 +63,24 @@ SIGNATURES = {
     "psa_density": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "psa_gather_rows": (c_int, [POINTER(Tensor4), POINTER(Tensor4), POINTER(c_int), c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                 c_void_p]),
+    "psa_pool_kv_indexed": (c_int, [Tensor4, Tensor4, c_void_p, Tensor4, Tensor4, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p]),
+    "psa_estimate_sampled_indexed": (
+        c_int,
+        [Tensor4, c_void_p, Tensor4, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_int, c_float, c_int, c_int, c_void_p],
+    ),
+    "psa_estimate_sampled_map_indexed": (
+        c_int,
+        [Tensor4, c_void_p, Tensor4, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_int, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int, c_int,
+         c_double, c_void_p],
+    ),
+    "psa_fwd_indexed": (
+        c_int,
+        [Tensor4, c_void_p, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,
+         c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
+    ),
     "psa_fwd": (
         c_int,
         [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,

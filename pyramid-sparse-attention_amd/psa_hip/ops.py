@@ -55,6 +55,31 @@ def pool_kv(k: torch.Tensor, v: torch.Tensor, block_n: int) -> Tuple[torch.Tenso
     return kp, vp
 
 
+def _check_index(index: torch.Tensor, L: int) -> torch.Tensor:
+    if index.dtype != torch.int32 or index.dim() != 1 or index.numel() != L:
+        raise ValueError("index must be a 1-D int32 tensor with one entry per token (%d)" % L)
+    return index.contiguous()
+
+
+def pool_kv_indexed(k: torch.Tensor, v: torch.Tensor, index: torch.Tensor, block_n: int):
+    """pool_kv of the re-ordered K, V (position i = source row index[i]; index an int32 permutation of 0..L-1) without a
+    gather pass of its own: returns (k_pool, v_pool, k_ord, v_ord), the last two being the re-ordered rows [B,H,L,D]."""
+    _require_gpu(k, v, index)
+    k, v = _bf16_view(k), _bf16_view(v)
+    B, H, L, D = k.shape
+    if v.shape != k.shape:
+        raise ValueError("k and v must have the same shape")
+    index = _check_index(index, L)
+    n = lib.psa_pool_elems(B, H, L, D, block_n)
+    kp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+    vp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+    ko, vo = torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
+    with torch.cuda.device(k.device):
+        check(lib.psa_pool_kv_indexed(_t4(k), _t4(v), _ptr(index), _t4(ko), _t4(vo), _ptr(kp), _ptr(vp), B, H, L, D, block_n,
+                                      _stream(k)), "psa_pool_kv_indexed")
+    return kp, vp, ko, vo
+
+
 def pool_levels(pool: torch.Tensor, B: int, H: int, L: int, D: int, block_n: int) -> Dict[int, torch.Tensor]:
     """Views [B,H,Npad/l,D] of the levels inside a pooled buffer."""
     npad = -(-L // block_n) * block_n
@@ -79,10 +104,12 @@ def estimate_sampled(
     sm_scale: Optional[float] = None,
     out_rows: Optional[int] = None,
     out_cols: Optional[int] = None,
+    q_index: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """fp32 block-importance scores [B,Hq,out_rows,out_cols]; off_* int32 [B,H,keep] in-block offsets
-    (None: rows are taken as 0..keep-1 of each block)."""
-    _require_gpu(q, k, off_q, off_k)
+    (None: rows are taken as 0..keep-1 of each block).  q_index (int32 permutation [Lq]): query position i is row
+    q_index[i] of q (token re-ordering read on the fly; k is passed already re-ordered)."""
+    _require_gpu(q, k, off_q, off_k, q_index)
     q, k = _bf16_view(q), _bf16_view(k)
     B, Hq, Lq, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
@@ -95,12 +122,14 @@ def estimate_sampled(
             raise ValueError("sample offsets must be contiguous int32 [B, H, keep]")
     scores = torch.empty(B, Hq, out_rows, out_cols, dtype=torch.float32, device=q.device)
     ws = torch.empty(lib.psa_estimate_workspace_bytes(B, Hq, Lq, Lk, block_m, block_n, keep_m, keep_n), dtype=torch.uint8, device=q.device)
+    tail = (_ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, float(sm_scale),
+            out_rows, out_cols, _stream(q))
     with torch.cuda.device(q.device):
-        check(
-            lib.psa_estimate_sampled(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D,
-                                     block_m, block_n, keep_m, keep_n, float(sm_scale), out_rows, out_cols, _stream(q)),
-            "psa_estimate_sampled",
-        )
+        if q_index is None:
+            check(lib.psa_estimate_sampled(_t4(q), _t4(k), *tail), "psa_estimate_sampled")
+        else:
+            check(lib.psa_estimate_sampled_indexed(_t4(q), _ptr(_check_index(q_index, Lq)), _t4(k), *tail),
+                  "psa_estimate_sampled_indexed")
     return scores
 
 
@@ -121,6 +150,7 @@ def estimate_sampled_map(
     map_dtype: torch.dtype = torch.int32,
     sm_scale: Optional[float] = None,
     return_scores: bool = False,
+    q_index: Optional[torch.Tensor] = None,
 ):
     """estimate_sampled + level_map (dense map modes, blocksize = block_n) with the map taken from each row of
     scores while it is still on chip: the same map, bit for bit, in two launches instead of three.  Returns the
@@ -130,7 +160,7 @@ def estimate_sampled_map(
         raise ValueError("the fused estimator writes dense maps only")
     if map_dtype not in (torch.int8, torch.int32):
         raise ValueError("map_dtype must be int8 or int32")
-    _require_gpu(q, k, off_q, off_k)
+    _require_gpu(q, k, off_q, off_k, q_index)
     q, k = _bf16_view(q), _bf16_view(k)
     B, Hq, Lq, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
@@ -150,13 +180,14 @@ def estimate_sampled_map(
     scores = torch.empty(B, Hq, Mq, Nk, dtype=torch.float32, device=q.device) if (return_scores or Nk > 4096) else None
     out = torch.empty(B, Hq, Mq, Nk, dtype=map_dtype, device=q.device)
     ws = torch.empty(lib.psa_estimate_workspace_bytes(B, Hq, Lq, Lk, block_m, block_n, keep_m, keep_n), dtype=torch.uint8, device=q.device)
+    tail = (_ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D, block_m, block_n, keep_m, keep_n, float(sm_scale),
+            Mq, Nk, _ptr(out), out.element_size(), m, n, lv, hi, div, tb, float(min_full_attn_ratio), _stream(q))
     with torch.cuda.device(q.device):
-        check(
-            lib.psa_estimate_sampled_map(_t4(q), _t4(k), _ptr(off_q), _ptr(off_k), _ptr(scores), _ptr(ws), B, Hq, Hkv, Lq, Lk, D,
-                                         block_m, block_n, keep_m, keep_n, float(sm_scale), Mq, Nk, _ptr(out), out.element_size(),
-                                         m, n, lv, hi, div, tb, float(min_full_attn_ratio), _stream(q)),
-            "psa_estimate_sampled_map",
-        )
+        if q_index is None:
+            check(lib.psa_estimate_sampled_map(_t4(q), _t4(k), *tail), "psa_estimate_sampled_map")
+        else:
+            check(lib.psa_estimate_sampled_map_indexed(_t4(q), _ptr(_check_index(q_index, Lq)), _t4(k), *tail),
+                  "psa_estimate_sampled_map_indexed")
     return (scores, out) if return_scores else out
 
 
@@ -352,11 +383,14 @@ def sparse_attention_fwd(
     pools: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
     out: Optional[torch.Tensor] = None,
     balance: bool = True,
+    q_index: Optional[torch.Tensor] = None,
 ):
     """Pyramid sparse attention forward.  level_map_ None = dense attention.  Returns out (dtype and
     shape of q) or (out, lse fp32 [B,H,L], (k_pool, v_pool)).  balance=True issues the rows of the map
-    longest first (same results, shorter tail)."""
-    _require_gpu(q, k, v, level_map_)
+    longest first (same results, shorter tail).  q_index (int32 permutation [L]): k, v, the pools and the map are in
+    the re-ordered token order, q is in the original order and read through the index (position i = row q_index[i]),
+    and out / lse come back in the original order (row q_index[i] = result of position i)."""
+    _require_gpu(q, k, v, level_map_, q_index)
     in_dtype = q.dtype
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     B, Hq, L, D = qb.shape
@@ -383,13 +417,13 @@ def sparse_attention_fwd(
     ws = None
     if level_map_ is not None and balance:
         ws = torch.empty(lib.psa_fwd_workspace_bytes(B, Hq, L, block_m) // 4, dtype=torch.int32, device=q.device)
+    tail = (_t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_), 1 if level_map_ is None else level_map_.element_size(), _t4(o),
+            _ptr(lse), B, Hq, Hkv, L, D, block_m, block_n, sm_scale, int(causal), _ptr(ws), _stream(q))
     with torch.cuda.device(q.device):
-        check(
-            lib.psa_fwd(_t4(qb), _t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_),
-                        1 if level_map_ is None else level_map_.element_size(), _t4(o), _ptr(lse), B, Hq, Hkv, L, D,
-                        block_m, block_n, sm_scale, int(causal), _ptr(ws), _stream(q)),
-            "psa_fwd",
-        )
+        if q_index is None:
+            check(lib.psa_fwd(_t4(qb), *tail), "psa_fwd")
+        else:
+            check(lib.psa_fwd_indexed(_t4(qb), _ptr(_check_index(q_index, L)), *tail), "psa_fwd_indexed")
     res = o if in_dtype == torch.bfloat16 else o.to(in_dtype)
     if return_lse:
         return res, lse, (kp, vp)
@@ -412,6 +446,7 @@ def psa_layer_fwd(
     level_cap: Optional[torch.Tensor] = None,
     return_map: bool = False,
     text_length: int = 0,
+    token_index: Optional[torch.Tensor] = None,
 ):
     """estimate (+ level map, in the estimator's reduction kernel) -> pooled K/V -> sparse attention, non-causal,
     no gradient: all on the current stream with a dense int8 level map in between (no index-list round trip).
@@ -421,12 +456,18 @@ def psa_layer_fwd(
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     keep_m, keep_n = block_m // 4, block_n // 4
     sm_scale = qb.shape[-1] ** -0.5 if sm_scale is None else float(sm_scale)
+    if token_index is not None:
+        # token re-ordering (int32 permutation: position i = source row token_index[i]) without gather passes: the pooling
+        # pass reads K, V through the index and leaves the re-ordered rows behind, the estimator and the attention kernel
+        # read Q through it, and the attention kernel writes its rows back to their original places
+        kp, vp, kb, vb = pool_kv_indexed(kb, vb, token_index, block_n)
     mp = estimate_sampled_map(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, mask_ratios, text_length, mode,
-                              compute_tile=tile_n, map_dtype=torch.int8, sm_scale=sm_scale)
+                              compute_tile=tile_n, map_dtype=torch.int8, sm_scale=sm_scale, q_index=token_index)
     if level_cap is not None:
         mp = map_min_cap(mp, level_cap)
-    kp, vp = pool_kv(kb, vb, block_n)
-    out = sparse_attention_fwd(qb, kb, vb, mp, block_m, block_n, sm_scale, pools=(kp, vp))
+    if token_index is None:
+        kp, vp = pool_kv(kb, vb, block_n)
+    out = sparse_attention_fwd(qb, kb, vb, mp, block_m, block_n, sm_scale, pools=(kp, vp), q_index=token_index)
     if out.dtype != q.dtype:
         out = out.to(q.dtype)
     return (out, mp) if return_map else out

@@ -63,8 +63,9 @@ class AttentionConfig:
             )
 
 
-def efficient_attn_with_pooling(q, k, v, config, num_keep_m=32, num_keep_n=32, sample_offsets=None):
-    """Block importance [B,H,Mq,Nk] fp32 and the similarity cap [B,H,Nk] (or None).
+def efficient_attn_with_pooling(q, k, v, config, num_keep_m=32, num_keep_n=32, sample_offsets=None, q_index=None):
+    """Block importance [B,H,Mq,Nk] fp32 and the similarity cap [B,H,Nk] (or None).  q_index: see
+    adaptive_block_sparse_attn.
     reference: src/psa_triton/pyramid_sparse_attention.py:139-187."""
     sim_cap = calc_k_similarity(k, config.block_n, config) if getattr(config, "use_sim_mask", True) else None
     B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
@@ -73,17 +74,23 @@ def efficient_attn_with_pooling(q, k, v, config, num_keep_m=32, num_keep_n=32, s
         off_k = draw_sample_offsets(B, Hkv, config.block_n, num_keep_n, k.device)
     else:
         off_q, off_k = sample_offsets
-    pooling = ops.estimate_sampled(q, k, off_q, off_k, config.block_m, config.block_n, num_keep_m, num_keep_n, q.size(-1) ** -0.5)
+    pooling = ops.estimate_sampled(q, k, off_q, off_k, config.block_m, config.block_n, num_keep_m, num_keep_n, q.size(-1) ** -0.5,
+                                   q_index=q_index)
     return pooling, sim_cap
 
 
-def adaptive_block_sparse_attn(q, k, v, config, sparse_attention_fn, compute_stats=False, sample_offsets=None):
+def adaptive_block_sparse_attn(q, k, v, config, sparse_attention_fn, compute_stats=False, sample_offsets=None, q_index=None,
+                               pools=None):
     """estimate -> mask (-> min with the similarity cap) -> sparse attention.
     Returns (out, sparsity, per_head_density, sim_cap); the statistics are device tensors
     (no host synchronisation) unless compute_stats is False, in which case they are 0.0 / [].
+    q_index / pools (token re-ordering without gather passes, forward only): k, v are the re-ordered rows and pools their
+    pooled levels (ops.pool_kv_indexed), q is in the original order and read through q_index, and out comes back in the
+    original order.
     reference: src/psa_triton/pyramid_sparse_attention.py:188-249."""
     with torch.no_grad():
-        pooling, sim_cap = efficient_attn_with_pooling(q, k, v, config, config.block_m // 4, config.block_n // 4, sample_offsets)
+        pooling, sim_cap = efficient_attn_with_pooling(q, k, v, config, config.block_m // 4, config.block_n // 4, sample_offsets,
+                                                       q_index)
         if config.attn_impl == "old_mask_type":
             mask = ops.level_map(pooling, config.mask_ratios, config.text_length, config.mask_mode, blocksize=config.block_n,
                                  compute_tile=config.tile_n)
@@ -95,9 +102,15 @@ def adaptive_block_sparse_attn(q, k, v, config, sparse_attention_fn, compute_sta
             raise ValueError(f"Unknown attn_impl: {config.attn_impl}")
         if getattr(config, "use_sim_mask", True) and sim_cap is not None:
             mask = ops.map_min_cap(mask, sim_cap)
-    out = sparse_attention_fn(q, k, v, mask, None)
+    dense = None
+    if q_index is None:
+        out = sparse_attention_fn(q, k, v, mask, None)
+    else:
+        dense = mask if config.attn_impl == "old_mask_type" else ops.map_from_list(mask, -(-k.shape[2] // config.block_n), torch.int8)
+        out = ops.sparse_attention_fwd(q, k, v, dense, config.block_m, config.block_n, pools=pools, q_index=q_index)
     if compute_stats:
-        dense = mask if config.attn_impl == "old_mask_type" else ops.map_from_list(mask, -(-k.shape[2] // config.block_n))
+        if dense is None:
+            dense = mask if config.attn_impl == "old_mask_type" else ops.map_from_list(mask, -(-k.shape[2] // config.block_n))
         d = ops.density(dense)  # [B*H + 1] on the device
         sparsity = 1 - d[-1]
         per_head = d[:-1].view(q.shape[0], q.shape[1]).mean(0)
@@ -128,6 +141,11 @@ class PyramidSparseAttention(nn.Module):
         self.sparsity_acc = 0.0
         self.sparsity_counter = 0
         self.use_rearrange = config.use_rearrange
+        # True: the re-ordering is read / written by the layer's own kernels through the token index (no gather passes);
+        # False: rearrange() before and reversed_rearrange() after, the reference's sequence of operations.  The two give
+        # the same bits outside the warm-up steps (during warm-up the first runs dense attention in the original order,
+        # which differs from the re-ordered dense attention only in the order of the fp32 sums over the keys).
+        self.fuse_rearrange = True
         self.inference_num = inference_num
         self.layer_num = layer_num
         self.sample_offsets = None
@@ -150,20 +168,29 @@ class PyramidSparseAttention(nn.Module):
         return (self.sparsity_counter // (2 * self.layer_num)) % self.inference_num
 
     def forward(self, q, k, v, layer_idx):
-        if self.rearranger is not None:
+        is_warmup = self.get_current_time() < self.config.warmup_steps
+        compute_stats = self.config.verbose or self.logger is not None
+        fused = (self.rearranger is not None and self.fuse_rearrange
+                 and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)))
+        restore = self.rearranger is not None and not fused
+        if restore:
             q_r, k_r, v_r = self.rearranger.rearrange(q, k, v)
         else:
             q_r, k_r, v_r = q, k, v
-        is_warmup = self.get_current_time() < self.config.warmup_steps
-        compute_stats = self.config.verbose or self.logger is not None
         sim_cap = None
         if is_warmup:
             out_r = ops.sparse_attention_fwd(q_r, k_r, v_r, None, 128, 128)  # dense attention, same kernel
             sparsity = 0.0
             per_head_density = [1.0] * q_r.shape[1] if compute_stats else []
         else:
+            index = pools = None
+            if fused:
+                index = self.rearranger.token_index(q.device)
+                kp, vp, k_r, v_r = ops.pool_kv_indexed(k, v, index, self.config.block_n)
+                pools = (kp, vp)
             out_r, sparsity, per_head_density, sim_cap = adaptive_block_sparse_attn(
-                q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets
+                q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets,
+                q_index=index, pools=pools
             )
             if compute_stats:
                 self.sparsity_acc = self.sparsity_acc + sparsity
@@ -172,7 +199,7 @@ class PyramidSparseAttention(nn.Module):
             self.logger.log_sparsity(layer_idx=layer_idx, sparsity=sparsity, per_head_density=per_head_density,
                                      sequence_length=q.shape[2], batch_size=q.shape[0], num_heads=q.shape[1], sim_mask=sim_cap,
                                      is_warmup=is_warmup)
-        return self.rearranger.reversed_rearrange(out_r) if self.rearranger is not None else out_r
+        return self.rearranger.reversed_rearrange(out_r) if restore else out_r
 
     def close_logger(self):
         if self.logger is not None:

@@ -46,6 +46,13 @@ class GilbertRearranger:
             self._cache[key] = idx.to(torch.int32).to(device)
         return self._cache[key]
 
+    def token_index(self, device) -> torch.Tensor:
+        """int32 [L]: position i of the re-ordered sequence (video tokens along the curve, then the text) is row
+        token_index[i] of the input.  The layer's kernels can read and write through it directly instead of calling
+        rearrange() / reversed_rearrange() (ops.pool_kv_indexed, the q_index arguments of the estimator and the
+        attention forward)."""
+        return self._combined_index(device, True)
+
     @staticmethod
     def _native(x: torch.Tensor) -> bool:
         # the HIP row gather handles GPU tensors [B, H, L, D] with 2- or 4-byte elements and 16-byte rows
