@@ -267,17 +267,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p)
   }
 }
 
-// slot -> (level, 64-key part inside the block); slots of a block: max(1, (bn>>lv)/64) per level
-__device__ __forceinline__ void decode_slot(int slot, int bn_log2, int& lv, int& part) {
-  lv = 0;
-  for (;;) {
-    const int n = (bn_log2 - lv) > 6 ? 1 << (bn_log2 - lv - 6) : 1;
-    if (slot < n) break;
-    slot -= n;
-    ++lv;
-  }
-  part = slot;
-}
+// slots of a kv-block in the dK/dV walk: one per level (a level-0 block of 128 keys is one slot of 128 keys)
+constexpr int DKDV_SLOTS = 4;
 
 // ------------------------------------------------------------------------------------------------------
 // Longest-columns-first order for the dK/dV walk.  A workgroup's work is the number of q-blocks that retain its
@@ -286,8 +277,10 @@ __device__ __forceinline__ void decode_slot(int slot, int bn_log2, int& lv, int&
 // ------------------------------------------------------------------------------------------------------
 constexpr int COL_BINS = 2048;
 
-// one workgroup per (kv head, kv-block): per-level counts over the column -> cost of each of its slots
-__global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int slots_per_block, int32_t* cost) {
+// one workgroup per (kv head, kv-block): per-level counts over the column -> cost of each of its slots.  The costs of
+// the slots slot_lo .. of all blocks form one list per dK/dV launch: with a 128-key slot 0 that slot's list comes first
+// (n_blocks entries), then the list of the slots 1 .. 3.
+__global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int wide0, int32_t* cost) {
   __shared__ int s_n[4];
   const int J = blockIdx.x, bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
   const int n_rep = p.Hq / p.Hkv, Mq = p.Mq, bn_log2 = p.bn_log2;
@@ -309,20 +302,28 @@ __global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int s
   for (int lv = 0; lv < 4; ++lv)
     if (n[lv]) atomicAdd(&s_n[lv], n[lv]);
   __syncthreads();
-  if ((int)threadIdx.x < slots_per_block) {
-    int lv, part;
-    decode_slot((int)threadIdx.x, bn_log2, lv, part);
-    const int c = s_n[lv];
-    cost[((int64_t)bhk * p.Nk + J) * slots_per_block + threadIdx.x] = c < COL_BINS - 1 ? c : COL_BINS - 1;
+  if ((int)threadIdx.x < DKDV_SLOTS) {
+    const int lv = (int)threadIdx.x;
+    const int c = s_n[lv] < COL_BINS - 1 ? s_n[lv] : COL_BINS - 1;
+    const int64_t blk = (int64_t)bhk * p.Nk + J, n_blocks = (int64_t)gridDim.y * p.Nk;
+    if (!wide0) cost[blk * DKDV_SLOTS + lv] = c;
+    else if (lv == 0) cost[blk] = c;
+    else cost[n_blocks + blk * (DKDV_SLOTS - 1) + (lv - 1)] = c;
   }
 }
 
 // one workgroup of 1024 threads: counting sort of all workgroup ids by decreasing cost
 constexpr int COLSORT_NT = 1024;
-__global__ __launch_bounds__(COLSORT_NT) void psa_bwd_colsort_kernel(const int32_t* cost, int total, int32_t* order) {
+__global__ __launch_bounds__(COLSORT_NT) void psa_bwd_colsort_kernel(const int32_t* cost, int total0, int total1, int32_t* order) {
   __shared__ int hist[COL_BINS];
   __shared__ int part[COLSORT_NT];
   const int tid = threadIdx.x;
+  // workgroup 0 sorts the first list (total0 entries), workgroup 1 the second one behind it; ids are list-local
+  const int total = blockIdx.x == 0 ? total0 : total1;
+  if (blockIdx.x == 1) {
+    cost += total0;
+    order += total0;
+  }
   for (int i = tid; i < COL_BINS; i += COLSORT_NT) hist[i] = 0;
   __syncthreads();
   for (int i = tid; i < total; i += COLSORT_NT) atomicAdd(&hist[cost[i]], 1);
@@ -357,11 +358,17 @@ __global__ __launch_bounds__(COLSORT_NT) void psa_bwd_colsort_kernel(const int32
 // buffered, one barrier per step of 64 query rows) in the padded + swizzled row-major tile layout of the forward
 // kernel; the row operands (S = Q K^T, dP = dO V^T) are 128-bit LDS reads and the transposed operands
 // (dV^T += dO^T P, dK^T += Q^T dS) come from the same tiles through the transposing LDS load.
+// The four waves of a workgroup split its keys and the 64 query rows of a step: 128 keys (level 0 of a 128-key
+// block) = 4 key quarters, every wave takes both query halves one after the other ("wide": each Q / dO tile that is
+// fetched feeds twice the arithmetic); <= 64 keys = 2 key halves x 2 query halves, combined through LDS at the end.
 // ------------------------------------------------------------------------------------------------------
 constexpr int B_ISTR = LT_ISTR;  // bytes between the blocks of a tile
 
-template <int D>
-__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slots_per_block, const int32_t* order) {
+// One instantiation per kind of slot (WIDE: the 128-key level-0 slot; else the slots slot_lo .. slot_lo + slot_cnt - 1 of
+// every kv-block); workgroup id = ((b * Hkv + kv head) * Nk + kv-block) * slot_cnt + (slot - slot_lo), optionally
+// re-ordered.
+template <int D, bool WIDE, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slot_lo, int slot_cnt, const int32_t* order) {
   using G = LtGeom<D>;
   constexpr int KK = D / 16, DB = D / 32, RPL = G::RPL;
   constexpr int B_TILE = G::TILE;
@@ -372,30 +379,30 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
   uint32_t* qlist = (uint32_t*)(s_del + 128);  // [n_rep * Mq]  (head in group << 16 | q-block)
   __shared__ int s_nq;
 
-  // flat workgroup id = ((b * Hkv + kv head) * Nk + kv-block) * slots_per_block + slot, optionally re-ordered
   const int wg = order != nullptr ? order[blockIdx.x] : (int)blockIdx.x;
-  const int slot = wg % slots_per_block;
-  const int J = (wg / slots_per_block) % p.Nk;
-  const int bhk = wg / (slots_per_block * p.Nk), b = bhk / p.Hkv, hk = bhk % p.Hkv;
+  const int slot = slot_lo + wg % slot_cnt;
+  const int J = (wg / slot_cnt) % p.Nk;
+  const int bhk = wg / (slot_cnt * p.Nk), b = bhk / p.Hkv, hk = bhk % p.Hkv;
   const int n_rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hh = lane >> 5;
   const int L = p.L, bn_log2 = p.bn_log2, causal = p.causal, bm = p.bm, Mq = p.Mq;
 
-  int lv, part;
-  decode_slot(slot, bn_log2, lv, part);
+  const int lv = slot;
   const int sbs = 1 << (bn_log2 - lv);            // pooled keys of this block at this level
-  const int nkeys = sbs < 64 ? sbs : 64;
-  const int64_t key_row0 = ((int64_t)J << (bn_log2 - lv)) + part * 64;  // first pooled row of this workgroup
+  constexpr bool wide = WIDE;                     // 128 keys (the host launches this instantiation for such slots only)
+  const int nkeys = sbs;
+  const int64_t key_row0 = (int64_t)J << (bn_log2 - lv);  // first pooled row of this workgroup
   int key_valid = nkeys;                          // level 0: rows past L do not exist
   if (lv == 0) {
     const int64_t rem = (int64_t)L - key_row0;
     key_valid = rem < nkeys ? (rem > 0 ? (int)rem : 0) : nkeys;
   }
-  // waves = 2 key halves x 2 query halves.  With at most 32 keys only one key half works: alternate which
-  // pair of waves that is from workgroup to workgroup, so that all four SIMDs of a CU get work.
+  // <= 64 keys: waves = 2 key halves x 2 query halves.  With at most 32 keys only one key half works: alternate
+  // which pair of waves that is from workgroup to workgroup, so that all four SIMDs of a CU get work.
+  // 128 keys: waves = 4 key quarters.
   const int flip = nkeys <= 32 ? (int)(blockIdx.x & 1) : 0;
-  const int kh = (wave & 1) ^ flip, qh = wave >> 1;
+  const int kh = wide ? wave : ((wave & 1) ^ flip), qh = wide ? 0 : wave >> 1;
   const bool wave_active = key_valid > kh * 32;
 
   // ---- list of (head in group, q-block) that retain block J at this level -------------------------
@@ -445,7 +452,6 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
       vf[kk] = *(const bf16x8*)(vp_ + kk * 16 + hh * 8);
     }
   }
-  const bool key_ok = key_local < key_valid;
   const int key_up = (int)(((key_row0 + key_local + 1) << lv) - 1);  // last token the pooled key covers (< npad)
   __syncthreads();
   const int nq = s_nq;
@@ -453,11 +459,15 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
   // ---- lane-invariant LDS addressing (tile layout: see the forward kernel) ---------------------------
   // copy: wave w fills the 16-row group w of both tiles; lane (fq = lane/16, pos = lane%16) of block n writes
   // row fq of that block, i.e. tile row 16w + 4fq + n, chunk pos ^ fq
-  const uint32_t f_chunk = lt_fetch_chunk<D>(lane);
-  const int f_row = wave * 16 + lt_fetch_row<D>(lane);
+  // (recomputed from the lane id at every use - see issue_step - instead of living in registers across the matrix work:
+  // this kernel has no register to spare, and a spilled value comes back through a vmcnt wait that would also wait
+  // for the tile copies in flight)
   uint32_t r_off[2], t_off[2];
+  // (qh = 0 in a wide workgroup, whose passes add HALF * query half as an immediate)
   lt_row_operand<D>(qh * 32 + l32, hh, r_off);  // row operand of k-step kk: r_off[kk & 1] + 64 * (kk >> 1)
-  lt_tr_operand<D>(lane, t_off);                // transposed operand: t_off[s] + 64 * db + 4 * B_ISTR * (16-row group)
+  lt_tr_operand<D>(lane, t_off);                // transposed operand: t_off[s] + 64 * db + GROUP * (16-row group)
+#pragma unroll
+  for (int i = 0; i < 2; ++i) t_off[i] += (uint32_t)(qh * G::HALF);
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -497,6 +507,10 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
     const char* qb = (const char*)(p.q + b * p.q_sb + h * p.q_sh);
     const char* ob = (const char*)(p.dout + b * p.do_sb + h * p.do_sh);
+    int ln = lane;
+    asm volatile("" : "+v"(ln));  // keeps the two values below out of the loop-invariant registers
+    const uint32_t f_chunk = lt_fetch_chunk<D>(ln);
+    const int f_row = wave * 16 + lt_fetch_row<D>(ln);
     const int r0 = q0 + f_row;
     if (q0 + 64 <= L) {
       const uint32_t qo = (uint32_t)r0 * q_strb + f_chunk, oo = (uint32_t)r0 * do_strb + f_chunk;
@@ -516,14 +530,15 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
       }
     }
   };
+  // (the level's bias goes in with the row's lse: one subtraction per row here instead of one per logit later)
   auto publish_rows = [&](int stage) __attribute__((always_inline)) {
     if (tid < 64) {
-      s_lse[stage * 64 + tid] = lse_next;
+      s_lse[stage * 64 + tid] = bias - lse_next;
       s_del[stage * 64 + tid] = del_next;
     }
   };
 
-  PSA_LDS(const float) rows_base = (PSA_LDS(const float))(smem + 4 * B_TILE) + (qh * 32 + hh * 4);
+  PSA_LDS(const float) rows_base0 = (PSA_LDS(const float))(smem + 4 * B_TILE) + (qh * 32 + hh * 4);
   auto compute_step = [&](int i, auto stage_c) __attribute__((always_inline)) {
     constexpr int ST = decltype(stage_c)::value;
     int h, I, q0;
@@ -531,8 +546,12 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     I = __builtin_amdgcn_readfirstlane(I);
     q0 = __builtin_amdgcn_readfirstlane(q0);
     const bool diag = causal && ((((int64_t)J + 1) << bn_log2) - 1 > (int64_t)I * bm);
-    PSA_LDS(unsigned char) Qs = (PSA_LDS(unsigned char))(smem) + 2 * ST * B_TILE;
-    PSA_LDS(unsigned char) Os = (PSA_LDS(unsigned char))(smem) + (2 * ST + 1) * B_TILE;
+#pragma unroll
+    for (int qi = 0; qi < (WIDE ? 2 : 1); ++qi) {
+    const int qhv = WIDE ? qi : qh;  // the query half of this pass (the lane offsets already hold qh)
+    PSA_LDS(unsigned char) Qs = (PSA_LDS(unsigned char))(smem) + 2 * ST * B_TILE + (WIDE ? qi * G::HALF : 0);
+    PSA_LDS(unsigned char) Os = (PSA_LDS(unsigned char))(smem) + (2 * ST + 1) * B_TILE + (WIDE ? qi * G::HALF : 0);
+    PSA_LDS(const float) rows_base = rows_base0 + (WIDE ? qi * 32 : 0);
     // S = Q K^T and dP = dO V^T for this wave's (32 q) x (32 keys): lane = key column, registers = q rows
     f32x16 s, dp;
 #pragma unroll
@@ -548,19 +567,23 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
       dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[kk], dp, 0, 0, 0);
     }
     uint32_t pk[8], dsk[8];
+    // p = exp2(scale * s + bias - lse), dS = p (dP - delta).  Lanes whose key does not exist (the ragged end of the
+    // sequence at level 0; lanes beyond the 16 keys of a level-8 block) work on a copy of the block's first key: the
+    // columns of dK^T / dV^T are independent of each other and those lanes' columns are never read.  Only the causal
+    // diagonal needs a mask: keys behind the query get p = 0 (thr: first query row of this pass, relative to the
+    // lane's rows, that sees the lane's key).
+    int thr = 0;
+    if (CAUSAL) thr = diag ? key_up - (q0 + qhv * 32 + hh * 4) : -0x40000000;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const int qq = qh * 32 + g * 8 + hh * 4;
-      // one lane base + immediates (stage, group, lse / delta array)
+      // one lane base + immediates (stage, group, bias - lse / delta array)
       const f32x4 l4 = *(PSA_LDS(const f32x4))(rows_base + ST * 64 + g * 8);
       const f32x4 d4 = *(PSA_LDS(const f32x4))(rows_base + 128 + ST * 64 + g * 8);
       float pv[4], dsv[4];
 #pragma unroll
       for (int e2 = 0; e2 < 4; ++e2) {
-        float pe = fast_exp2(__builtin_fmaf(s[g * 4 + e2], scale_log2, bias - l4[e2]));
-        bool ok = key_ok;
-        if (diag) ok = ok && (key_up <= q0 + qq + e2);
-        pe = ok ? pe : 0.f;
+        float pe = fast_exp2(__builtin_fmaf(s[g * 4 + e2], scale_log2, l4[e2]));
+        if (CAUSAL) pe = thr <= g * 8 + e2 ? pe : 0.f;
         pv[e2] = pe;
         dsv[e2] = pe * (dp[g * 4 + e2] - d4[e2]);
       }
@@ -575,7 +598,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
       u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
       u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
       const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
-      const int grp = (2 * qh + g) * G::GROUP;
+      const int grp = g * G::GROUP;  // (Qs, Os already point at this pass's query half = two 16-row groups)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const u32x2 olo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[0] + db * 64 + grp)));
@@ -587,6 +610,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
         u32x4 qa2 = {qlo[0], qlo[1], qhi[0], qhi[1]};
         dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qa2), sfrag, dk[db], 0, 0, 0);
       }
+    }
+    if (WIDE) __builtin_amdgcn_sched_barrier(0);  // the second pass starts after the first: its operands do not fit beside it
     }
   };
 
@@ -614,10 +639,10 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
   }
 
-  // ---- combine the two query halves and write this workgroup's rows of the level buffers ------------
+  // ---- combine the two query halves (<= 64 keys) and write this workgroup's rows of the level buffers ----
   __syncthreads();
   float* red = (float*)smem;  // [2 key halves][2 tensors][DB*16][64 lanes]
-  if (qh == 1) {
+  if (!wide && qh == 1) {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -642,8 +667,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
 #pragma unroll
         for (int e2 = 0; e2 < 4; ++e2) {
           const int i = g * 4 + e2;
-          a[e2] = (dk[db][i] + red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane]) * scale;
-          c2[e2] = dv[db][i] + red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane];
+          a[e2] = (dk[db][i] + (wide ? 0.f : red[((kh * 2 + 0) * DB * 16 + db * 16 + i) * 64 + lane])) * scale;
+          c2[e2] = dv[db][i] + (wide ? 0.f : red[((kh * 2 + 1) * DB * 16 + db * 16 + i) * 64 + lane]);
         }
         *(f32x4*)(wk + db * 32 + g * 8 + hh * 4) = a;
         *(f32x4*)(wv + db * 32 + g * 8 + hh * 4) = c2;
@@ -699,11 +724,6 @@ __global__ __launch_bounds__(256) void psa_bwd_unpool_kernel(BwdParams p, int D)
   *(u32x2*)(dst + c * 4) = o;
 }
 
-int slots_of(int block_n) {
-  int n = 0;
-  for (int lv = 0; lv < 4; ++lv) n += (block_n >> lv) > 64 ? (block_n >> lv) / 64 : 1;
-  return n;
-}
 
 }  // namespace
 
@@ -799,32 +819,57 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     rc = psa_check_launch("psa_bwd (dQ)");
     if (rc != PSA_OK) return rc;
   }
-  // 3. dK, dV per level
+  // 3. dK, dV per level: the 128-key level-0 slots (if block_n = 128) in one launch, the other slots in a second one
   {
-    const int spb = slots_of(block_n);
     const int n_rep = Hq / Hkv;
-    const int64_t n_wg = (int64_t)B * Hkv * Nk * spb;
-    PSA_REQUIRE(n_wg < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    const bool wide0 = block_n > 64;
+    const int64_t n_blocks = (int64_t)B * Hkv * Nk;
+    const int64_t n_wide = wide0 ? n_blocks : 0, n_rest = n_blocks * (wide0 ? DKDV_SLOTS - 1 : DKDV_SLOTS);
+    PSA_REQUIRE(n_wide + n_rest < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
     size_t shmem = (size_t)4 * (D == 128 ? LtGeom<128>::TILE : LtGeom<64>::TILE) + 256 * sizeof(float) + (size_t)n_rep * Mq * 4;
     const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
     if (shmem < red) shmem = red;
     PSA_REQUIRE(shmem <= 160 * 1024, PSA_ERR_UNSUPPORTED, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
-    // longest columns first (needs a level map; the order lives behind lse2 in the workspace)
-    int32_t* order = nullptr;
-    if (map != nullptr && n_wg > 32) {
+    // longest columns first per launch (needs a level map; costs and orders live behind lse2 in the workspace)
+    int32_t *order_wide = nullptr, *order_rest = nullptr;
+    if (map != nullptr && n_blocks > 8) {
       int32_t* cost = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
-      order = cost + n_wg;
-      hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, spb, cost);
+      int32_t* order = cost + (n_wide + n_rest);
+      hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, wide0 ? 1 : 0, cost);
       if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
-      hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(COLSORT_NT), 0, st, cost, (int)n_wg, order);
+      if (wide0) {
+        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(2), dim3(COLSORT_NT), 0, st, cost, (int)n_wide, (int)n_rest, order);
+        order_wide = order;
+        order_rest = order + n_wide;
+      } else {
+        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(COLSORT_NT), 0, st, cost, (int)n_rest, 0, order);
+        order_rest = order;
+      }
       if (int e = psa_check_launch("psa_bwd (column order)")) return e;
     }
-    auto launch = [&](auto kern) -> int {
+    auto launch = [&](auto kern, int64_t n_wg, int slot_lo, int slot_cnt, const int32_t* order) -> int {
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) return PSA_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3(256), shmem, st, p, spb, order);
+      hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3(256), shmem, st, p, slot_lo, slot_cnt, order);
       return PSA_OK;
     };
-    const int rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128>) : launch(psa_bwd_dkdv_lds_kernel<64>);
+    int rl = PSA_OK;
+    if (wide0) {
+      if (causal)
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true>, n_wide, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, true>, n_wide, 0, 1, order_wide);
+      else
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false>, n_wide, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, false>, n_wide, 0, 1, order_wide);
+      PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
+      if (int e = psa_check_launch("psa_bwd (dK/dV, 128-key slots)")) return e;
+    }
+    const int lo = wide0 ? 1 : 0;
+    if (causal)
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, lo, DKDV_SLOTS - lo, order_rest);
+    else
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, lo, DKDV_SLOTS - lo, order_rest);
     PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
     const int rc = psa_check_launch("psa_bwd (dK/dV)");
     if (rc != PSA_OK) return rc;

@@ -40,6 +40,18 @@ namespace {
 #define PSA_FWD_ONE_GROUP 0
 #endif
 constexpr int TK = 64;              // pooled keys per tile
+template <int V>
+using IC = std::integral_constant<int, V>;
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(IC<Is>{}), ...);
+}
+// f(IC<0>{}), ..., f(IC<N-1>{}): a loop whose index is a compile-time constant in the body
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 constexpr float LAZY_THRESHOLD = 8.f;  // log2 units the running max may lag behind
 
 struct FwdParams {
@@ -550,8 +562,11 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     return r;
   };
   // One copy instruction: block n of this wave's 16-row group, into the tile buffer at byte lds_byte of the group
-  auto issue_one = [&](const char* base, uint32_t str, int row, int lds_byte, int n) __attribute__((always_inline)) {
-    psa_tiles::lds_copy16(base, __umul24((uint32_t)row, str) + f_chunk, psa_tiles::lds_addr_of(smem + lds_byte + (wave * G::RPL + n) * F_ISTR));
+  // One copy instruction: block N of this wave's 16-row group, into the tile buffer at byte LDS_BYTE of the group
+  // (the group's and the wave's part of the address as one integer: no null test per address derived from it)
+  const uint32_t wave_lds = psa_tiles::lds_addr_of(smem) + (uint32_t)(wave * G::RPL * F_ISTR);
+  auto issue_one = [&](const char* base, uint32_t str, int row, auto lds_byte, auto n) __attribute__((always_inline)) {
+    psa_tiles::lds_copy16_row<decltype(lds_byte)::value + decltype(n)::value * F_ISTR>(base, (uint32_t)row, str, f_chunk, wave_lds);
   };
   // The matrix work of one phase: S^T = K Q^T (tile in K buffer KB) and then O^T += V^T P^T (tile in V buffer
   // 1 - KB, probabilities pk2).  Only one wave per SIMD is in its matrix phase, so nothing else hides the LDS
@@ -691,10 +706,10 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       float lsum = 0.f;
       int n_lv = 0, n_sbs = 0, n_g = 0, n_lim = 0;
       uint16_t n_id = 0;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        if (c < 4) issue_one(ts.vbase, ts.vstr, ts.row[c], (2 + (CUR ^ 1)) * F_TILE, c);
-        else issue_one(ts2.kbase, ts2.kstr, ts2.row[c - 4], CUR * F_TILE, c - 4);
+      static_for<8>([&](auto cc) __attribute__((always_inline)) {
+        constexpr int c = decltype(cc)::value;
+        if constexpr (c < 4) issue_one(ts.vbase, ts.vstr, ts.row[c], IC<(2 + (CUR ^ 1)) * F_TILE>{}, IC<c>{});
+        else issue_one(ts2.kbase, ts2.kstr, ts2.row[c - 4], IC<CUR * F_TILE>{}, IC<c - 4>{});
         prob4(s[c >> 2], (c & 3) * 4, nb, pk[c >> 2] + (c & 3) * 2, lsum);
         if (c == 0) {
           const uint32_t d0 = __builtin_amdgcn_readfirstlane(dd2[0]), d1 = __builtin_amdgcn_readfirstlane(dd2[1]);
@@ -720,7 +735,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
           for (int n = 0; n < G::RPL; ++n) ts2.row[n] = src0 + n < n_lim ? src0 + n : n_lim;
         }
         __builtin_amdgcn_sched_barrier(0);
-      }
+      });
       ts = ts2;
       l_run = l_run * alpha + lsum;
     }

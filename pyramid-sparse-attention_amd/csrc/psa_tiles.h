@@ -318,6 +318,20 @@ __device__ __forceinline__ void lds_copy16(const char* sbase, uint32_t voff, uin
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
+// the same with the target given as a uniform LDS address plus a compile-time byte offset (M0 = lds_base + OFF in one
+// scalar instruction) and the lane offset row * str + chunk computed between the write of M0 and the copy (the
+// instruction that the hardware needs between the two anyway): three instructions per copy
+template <int OFF>
+__device__ __forceinline__ void lds_copy16_row(const char* sbase, uint32_t row, uint32_t str, uint32_t chunk, uint32_t lds_base) {
+  sbase = uniform_ptr(sbase);
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  str = __builtin_amdgcn_readfirstlane(str);
+  uint32_t voff;
+  asm volatile("s_add_u32 m0, %1, %6\n\tv_mad_u32_u24 %0, %2, %3, %4\n\tglobal_load_lds_dwordx4 %0, %5"
+               : "=&v"(voff)
+               : "s"(lds_base), "v"(row), "s"(str), "v"(chunk), "s"(sbase), "n"(OFF)
+               : "memory", "scc");
+}
 // the same with a full per-lane address
 __device__ __forceinline__ void lds_copy16_addr(const char* vaddr, uint32_t lds_addr) {
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
