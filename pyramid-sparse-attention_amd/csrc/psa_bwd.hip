@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "psa_tiles.h"
+#include "psa_order.h"
 
 namespace {
 
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
 // read them row-wise (128-bit reads), dQ^T += K^T dS^T reads the K tile through the transposing LDS load.
 // ------------------------------------------------------------------------------------------------------
 template <int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p) {
+__global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p, int chunk, const int32_t* order) {
   using G = LtGeom<D>;
   constexpr int LT_TILE = G::TILE;
   constexpr int NT = NW * 64, BM = NW * 32, CH = D / 8, KK = D / 16, DB = D / 32;
@@ -89,8 +90,12 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p)
   uint16_t* ids = (uint16_t*)(tdesc + p.max_tiles);
   __shared__ int s_cnt[4], s_ioff[4], s_toff[5], s_wcnt[4 * NW];
 
-  const int I = blockIdx.x % p.Mq;
-  const int bh = blockIdx.x / p.Mq;
+  // the workgroup's row (b, h, q-block): shares of rows per XCD, longest rows first (see psa_order.h)
+  int row = psa_order::dealt_entry((int)blockIdx.x, chunk);
+  if (order != nullptr) row = order[row];
+  if (row < 0 || row >= p.B * p.Hq * p.Mq) return;
+  const int I = row % p.Mq;
+  const int bh = row / p.Mq;
   const int h = bh % p.Hq, b = bh / p.Hq;
   const int hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -275,7 +280,7 @@ constexpr int DKDV_SLOTS = 4;
 // kv-block at its level, which varies a lot (a few key blocks are kept by every query block); issuing the
 // workgroups by decreasing work removes the tail of the launch.  Results do not depend on the order.
 // ------------------------------------------------------------------------------------------------------
-constexpr int COL_BINS = 2048;
+constexpr int COL_BINS = psa_order::COST_BINS;
 
 // one workgroup per (kv head, kv-block): per-level counts over the column -> cost of each of its slots.  The costs of
 // the slots slot_lo .. of all blocks form one list per dK/dV launch: with a 128-key slot 0 that slot's list comes first
@@ -312,47 +317,6 @@ __global__ __launch_bounds__(256) void psa_bwd_colcost_kernel(BwdParams p, int w
   }
 }
 
-// one workgroup of 1024 threads: counting sort of all workgroup ids by decreasing cost
-constexpr int COLSORT_NT = 1024;
-__global__ __launch_bounds__(COLSORT_NT) void psa_bwd_colsort_kernel(const int32_t* cost, int total0, int total1, int32_t* order) {
-  __shared__ int hist[COL_BINS];
-  __shared__ int part[COLSORT_NT];
-  const int tid = threadIdx.x;
-  // workgroup 0 sorts the first list (total0 entries), workgroup 1 the second one behind it; ids are list-local
-  const int total = blockIdx.x == 0 ? total0 : total1;
-  if (blockIdx.x == 1) {
-    cost += total0;
-    order += total0;
-  }
-  for (int i = tid; i < COL_BINS; i += COLSORT_NT) hist[i] = 0;
-  __syncthreads();
-  for (int i = tid; i < total; i += COLSORT_NT) atomicAdd(&hist[cost[i]], 1);
-  __syncthreads();
-  constexpr int PER = COL_BINS / COLSORT_NT;  // thread i owns the bins COL_BINS-1-PER*i .. COL_BINS-PER-PER*i
-  int c[PER], sum = 0;
-#pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    c[j] = hist[COL_BINS - 1 - (tid * PER + j)];
-    sum += c[j];
-  }
-  part[tid] = sum;
-  __syncthreads();
-  for (int d = 1; d < COLSORT_NT; d <<= 1) {
-    const int add = tid >= d ? part[tid - d] : 0;
-    __syncthreads();
-    part[tid] += add;
-    __syncthreads();
-  }
-  int run = part[tid] - sum;
-#pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    hist[COL_BINS - 1 - (tid * PER + j)] = run;
-    run += c[j];
-  }
-  __syncthreads();
-  for (int i = tid; i < total; i += COLSORT_NT) order[atomicAdd(&hist[cost[i]], 1)] = i;
-}
-
 // ------------------------------------------------------------------------------------------------------
 // dK/dV column walk, head dim 128: Q and dO rows are copied from global memory straight into LDS (double
 // buffered, one barrier per step of 64 query rows) in the padded + swizzled row-major tile layout of the forward
@@ -368,7 +332,8 @@ constexpr int B_ISTR = LT_ISTR;  // bytes between the blocks of a tile
 // every kv-block); workgroup id = ((b * Hkv + kv head) * Nk + kv-block) * slot_cnt + (slot - slot_lo), optionally
 // re-ordered.
 template <int D, bool WIDE, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slot_lo, int slot_cnt, const int32_t* order) {
+__global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slot_lo, int slot_cnt, int n_wg, int chunk,
+                                                                 const int32_t* order) {
   using G = LtGeom<D>;
   constexpr int KK = D / 16, DB = D / 32, RPL = G::RPL;
   constexpr int B_TILE = G::TILE;
@@ -379,7 +344,9 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
   uint32_t* qlist = (uint32_t*)(s_del + 128);  // [n_rep * Mq]  (head in group << 16 | q-block)
   __shared__ int s_nq;
 
-  const int wg = order != nullptr ? order[blockIdx.x] : (int)blockIdx.x;
+  int wg = psa_order::dealt_entry((int)blockIdx.x, chunk);  // shares of slots per XCD, longest lists first (psa_order.h)
+  if (order != nullptr) wg = order[wg];
+  if (wg < 0 || wg >= n_wg) return;
   const int slot = slot_lo + wg % slot_cnt;
   const int J = (wg / slot_cnt) % p.Nk;
   const int bhk = wg / (slot_cnt * p.Nk), b = bhk / p.Hkv, hk = bhk % p.Hkv;
@@ -401,7 +368,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
   // <= 64 keys: waves = 2 key halves x 2 query halves.  With at most 32 keys only one key half works: alternate
   // which pair of waves that is from workgroup to workgroup, so that all four SIMDs of a CU get work.
   // 128 keys: waves = 4 key quarters.
-  const int flip = nkeys <= 32 ? (int)(blockIdx.x & 1) : 0;
+  const int flip = nkeys <= 32 ? (int)((blockIdx.x >> 3) & 1) : 0;
   const int kh = wide ? wave : ((wave & 1) ^ flip), qh = wide ? 0 : wave >> 1;
   const bool wave_active = key_valid > kh * 32;
 
@@ -731,9 +698,10 @@ extern "C" int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D,
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || L <= 0 || D <= 0 || block_n <= 0) return 0;
   const int64_t npad = (int64_t)((L + block_n - 1) / block_n) * block_n;
   const int64_t levels = (int64_t)B * Hkv * D * (npad + npad / 2 + npad / 4 + npad / 8);
-  // + cost and order of the dK/dV workgroups (at most 8 slots per kv-block)
-  const int64_t n_wg = (int64_t)B * Hkv * ((L + block_n - 1) / block_n) * 8;
-  return (2 * levels + 2 * (int64_t)B * Hq * L + 2 * n_wg) * (int64_t)sizeof(float);
+  // + cost and issue order of the dQ rows (block_m >= 64) and of the dK/dV slots (4 per kv-block), padded to whole shares
+  const int64_t pad = 16 * psa_order::MAX_PHASES;
+  const int64_t n_rows = (int64_t)B * Hq * ((L + 63) / 64), n_slots = (int64_t)B * Hkv * ((L + block_n - 1) / block_n) * DKDV_SLOTS;
+  return (2 * levels + 2 * (int64_t)B * Hq * L + 2 * (n_rows + pad) + 2 * (n_slots + 2 * pad)) * (int64_t)sizeof(float);
 }
 
 extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool, const void* map,
@@ -798,16 +766,33 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     const int rc = psa_check_launch("psa_bwd (delta)");
     if (rc != PSA_OK) return rc;
   }
+  // issue orders (costs and orders live behind lse2 in the workspace; every list is padded to whole shares)
+  int32_t* ws_int = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
   // 2. dQ
   {
     const int64_t total = (int64_t)B * Hq * Mq;
-    PSA_REQUIRE(total < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    PSA_REQUIRE(total < (1ll << 28), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    int chunk, groups;
+    const double kv_bytes = 2.0 * B * Hkv * (double)p.npad * D * 2.0 * (map != nullptr ? 1.875 : 1.0);
+    psa_order::deal(total, kv_bytes, B * Hkv, chunk, groups);
+    const int32_t* order = nullptr;
+    if (map != nullptr && total > 8 * 32) {
+      int32_t* cost = ws_int;
+      int32_t* ord = cost + total;
+      hipLaunchKernelGGL(psa_order::psa_row_cost_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, st, map, map_elem_bytes, (int)total,
+                         Mq, Nk, p.bn_log2, block_m, p.causal, cost);
+      if (int e = psa_check_launch("psa_bwd (row cost)")) return e;
+      hipLaunchKernelGGL(psa_order::psa_chunk_sort_kernel, dim3((unsigned)groups), dim3(256), 0, st, cost, (int)total, chunk, ord);
+      if (int e = psa_check_launch("psa_bwd (row order)")) return e;
+      order = ord;
+    }
+    ws_int += 2 * total + 16 * psa_order::MAX_PHASES;
     auto launch = [&](auto kern, size_t tile_bytes, int nw) -> int {
       const size_t shmem = tile_bytes + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
       if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
       if (shmem > 48 * 1024 && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
         return PSA_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(nw * 64), shmem, st, p);
+      hipLaunchKernelGGL(kern, dim3((unsigned)(chunk * groups)), dim3(nw * 64), shmem, st, p, chunk, order);
       return PSA_OK;
     };
     int rc;
@@ -825,51 +810,55 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     const bool wide0 = block_n > 64;
     const int64_t n_blocks = (int64_t)B * Hkv * Nk;
     const int64_t n_wide = wide0 ? n_blocks : 0, n_rest = n_blocks * (wide0 ? DKDV_SLOTS - 1 : DKDV_SLOTS);
-    PSA_REQUIRE(n_wide + n_rest < (1ll << 30), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
+    PSA_REQUIRE(n_wide + n_rest < (1ll << 28), PSA_ERR_UNSUPPORTED, "psa_bwd: too many workgroups");
     size_t shmem = (size_t)4 * (D == 128 ? LtGeom<128>::TILE : LtGeom<64>::TILE) + 256 * sizeof(float) + (size_t)n_rep * Mq * 4;
     const size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
     if (shmem < red) shmem = red;
     PSA_REQUIRE(shmem <= 160 * 1024, PSA_ERR_UNSUPPORTED, "psa_bwd: too many q-blocks for the on-chip lists (LDS)");
-    // longest columns first per launch (needs a level map; costs and orders live behind lse2 in the workspace)
-    int32_t *order_wide = nullptr, *order_rest = nullptr;
+    // shares by the Q / dO rows the walk streams
+    const double qdo_bytes = 2.0 * B * Hq * (double)L * D * 2.0;
+    int chunk_w = 1, groups_w = 8, chunk_r, groups_r;
+    if (wide0) psa_order::deal(n_wide, qdo_bytes, B * Hkv, chunk_w, groups_w);
+    psa_order::deal(n_rest, qdo_bytes, B * Hkv, chunk_r, groups_r);
+    const int32_t *order_wide = nullptr, *order_rest = nullptr;
     if (map != nullptr && n_blocks > 8) {
-      int32_t* cost = (int32_t*)(p.lse2 + (int64_t)B * Hq * L);
-      int32_t* order = cost + (n_wide + n_rest);
+      int32_t* cost = ws_int;
+      int32_t* ord_w = cost + (n_wide + n_rest);
+      int32_t* ord_r = ord_w + (wide0 ? (int64_t)chunk_w * groups_w : 0);
       hipLaunchKernelGGL(psa_bwd_colcost_kernel, dim3((unsigned)Nk, (unsigned)(B * Hkv)), dim3(256), 0, st, p, wide0 ? 1 : 0, cost);
       if (int e = psa_check_launch("psa_bwd (column cost)")) return e;
       if (wide0) {
-        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(2), dim3(COLSORT_NT), 0, st, cost, (int)n_wide, (int)n_rest, order);
-        order_wide = order;
-        order_rest = order + n_wide;
-      } else {
-        hipLaunchKernelGGL(psa_bwd_colsort_kernel, dim3(1), dim3(COLSORT_NT), 0, st, cost, (int)n_rest, 0, order);
-        order_rest = order;
+        hipLaunchKernelGGL(psa_order::psa_chunk_sort_kernel, dim3((unsigned)groups_w), dim3(256), 0, st, cost, (int)n_wide, chunk_w, ord_w);
+        order_wide = ord_w;
       }
+      hipLaunchKernelGGL(psa_order::psa_chunk_sort_kernel, dim3((unsigned)groups_r), dim3(256), 0, st, cost + n_wide, (int)n_rest, chunk_r,
+                         ord_r);
+      order_rest = ord_r;
       if (int e = psa_check_launch("psa_bwd (column order)")) return e;
     }
-    auto launch = [&](auto kern, int64_t n_wg, int slot_lo, int slot_cnt, const int32_t* order) -> int {
+    auto launch = [&](auto kern, int64_t n_wg, int chunk, int groups, int slot_lo, int slot_cnt, const int32_t* order) -> int {
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) return PSA_ERR_LAUNCH;
-      hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3(256), shmem, st, p, slot_lo, slot_cnt, order);
+      hipLaunchKernelGGL(kern, dim3((unsigned)(chunk * groups)), dim3(256), shmem, st, p, slot_lo, slot_cnt, (int)n_wg, chunk, order);
       return PSA_OK;
     };
     int rl = PSA_OK;
     if (wide0) {
       if (causal)
-        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true>, n_wide, 0, 1, order_wide)
-                      : launch(psa_bwd_dkdv_lds_kernel<64, true, true>, n_wide, 0, 1, order_wide);
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, true>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
       else
-        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false>, n_wide, 0, 1, order_wide)
-                      : launch(psa_bwd_dkdv_lds_kernel<64, true, false>, n_wide, 0, 1, order_wide);
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
       PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
       if (int e = psa_check_launch("psa_bwd (dK/dV, 128-key slots)")) return e;
     }
     const int lo = wide0 ? 1 : 0;
     if (causal)
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, lo, DKDV_SLOTS - lo, order_rest);
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
     else
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, lo, DKDV_SLOTS - lo, order_rest);
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
     PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
     const int rc = psa_check_launch("psa_bwd (dK/dV)");
     if (rc != PSA_OK) return rc;

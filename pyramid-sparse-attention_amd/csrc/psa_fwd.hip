@@ -33,6 +33,7 @@
 
 #include "psa_common.h"
 #include "psa_tiles.h"
+#include "psa_order.h"
 
 namespace {
 
@@ -786,82 +787,6 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   }
 }
 
-// ---- longest-rows-first ordering ---------------------------------------------------------------------
-// Rows of the level map differ in the number of tiles they retain.  Workgroup ids are dealt round-robin
-// to the 8 XCDs and each XCD runs its ids in order, so sorting every XCD's share by decreasing tile count
-// shortens the tail of the launch.  The order only changes WHEN a row is computed, never its result.
-constexpr int COST_BINS = 2048;
-constexpr int FWD_MAX_PHASES = 64;
-constexpr int64_t FWD_PHASE_BYTES = 128ll << 20;  // K/V (+ pooled levels) in use at one time
-
-__global__ __launch_bounds__(256) void psa_fwd_cost_kernel(const void* map, int map_elem, int total, int Mq, int Nk, int bn_log2,
-                                                         int bm, int causal, int32_t* cost) {
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (row >= total) return;
-  const int I = row % Mq;
-  int jmax = Nk;
-  if (causal) {
-    const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
-    jmax = ce < jmax ? ce : jmax;
-  }
-  int cnt[4] = {0, 0, 0, 0};
-  for (int j0 = 0; j0 < jmax; j0 += 64) {
-    const int j = j0 + lane;
-    const int lvl = j < jmax ? load_map(map, (int64_t)row * Nk + j, map_elem) : 0;
-#pragma unroll
-    for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
-  }
-  if (lane == 0) {
-    int tiles = 0;
-#pragma unroll
-    for (int lv = 0; lv < 4; ++lv) tiles += ((cnt[lv] << (bn_log2 - lv)) + 63) >> 6;
-    cost[row] = tiles < COST_BINS - 1 ? tiles : COST_BINS - 1;
-  }
-}
-
-// one workgroup per group of rows: counting sort by decreasing cost
-__global__ __launch_bounds__(256) void psa_fwd_sort_kernel(const int32_t* cost, int total, int chunk, int32_t* order) {
-  __shared__ int hist[COST_BINS];
-  const int x = blockIdx.x, tid = threadIdx.x;
-  const int r0 = x * chunk;
-  for (int i = tid; i < COST_BINS; i += 256) hist[i] = 0;
-  __syncthreads();
-  for (int i = tid; i < chunk; i += 256)
-    if (r0 + i < total) atomicAdd(&hist[cost[r0 + i]], 1);
-  __syncthreads();
-  {  // start offset of every bin, highest cost first: thread i owns the 8 bins COST_BINS-1-8i .. COST_BINS-8-8i
-    __shared__ int part[256];
-    constexpr int PER = COST_BINS / 256;
-    int c[PER], sum = 0;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      c[j] = hist[COST_BINS - 1 - (tid * PER + j)];
-      sum += c[j];
-    }
-    part[tid] = sum;
-    __syncthreads();
-    for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the threads
-      const int add = tid >= d ? part[tid - d] : 0;
-      __syncthreads();
-      part[tid] += add;
-      __syncthreads();
-    }
-    int run = part[tid] - sum;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      hist[COST_BINS - 1 - (tid * PER + j)] = run;
-      run += c[j];
-    }
-  }
-  __syncthreads();
-  for (int i = tid; i < chunk; i += 256) {
-    if (r0 + i < total) order[r0 + atomicAdd(&hist[cost[r0 + i]], 1)] = r0 + i;
-  }
-  // ids past the last row of the last share
-  const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;
-  for (int i = valid + tid; i < chunk; i += 256) order[r0 + i] = -1;
-}
-
 template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
@@ -894,7 +819,7 @@ size_t pp_lds_bytes(int max_tiles, int Nk) {
 extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
   if (B <= 0 || Hq <= 0 || L <= 0 || block_m <= 0) return 0;
   const int64_t total = (int64_t)B * Hq * ((L + block_m - 1) / block_m);
-  return 2 * (total + 16 * FWD_MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
+  return 2 * (total + 16 * psa_order::MAX_PHASES) * (int64_t)sizeof(int32_t);  // any grouping of the rows fits
 }
 
 static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
@@ -936,15 +861,10 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
   p.total_wg = (int)total;
   // Groups of rows run one after the other on each XCD.  With several phases (8 groups each) the K/V of only a
   // few heads is in use at a time, so that the part of it that misses L2 can stay in the last-level cache.
-  int phases = 1;
   {
     const double kv_bytes = 2.0 * B * Hkv * ((double)Nk * block_n) * D * 2.0 * (map != nullptr ? 1.875 : 1.0);
-    phases = (int)(kv_bytes / (double)FWD_PHASE_BYTES) + 1;
-    const int max_phases = B * Hkv < FWD_MAX_PHASES ? B * Hkv : FWD_MAX_PHASES;
-    phases = phases > max_phases ? max_phases : phases;
+    psa_order::deal(total, kv_bytes, B * Hkv, p.wg_chunk, p.wg_groups);
   }
-  p.wg_groups = 8 * phases;
-  p.wg_chunk = (int)((total + p.wg_groups - 1) / p.wg_groups);
   // worst case: every kv-block at level 1, plus one partly filled tile per pooled level
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
   p.grp_bytes = 0;
@@ -959,10 +879,10 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
     PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
     int32_t* order = (int32_t*)workspace;
     int32_t* cost = order + (int64_t)p.wg_chunk * p.wg_groups;
-    hipLaunchKernelGGL(psa_fwd_cost_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes,
+    hipLaunchKernelGGL(psa_order::psa_row_cost_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, (hipStream_t)stream, map, map_elem_bytes,
                        (int)total, Mq, Nk, p.bn_log2, block_m, p.causal, cost);
     if (int e = psa_check_launch("psa_fwd (row cost)")) return e;
-    hipLaunchKernelGGL(psa_fwd_sort_kernel, dim3(p.wg_groups), dim3(256), 0, (hipStream_t)stream, cost, (int)total, p.wg_chunk, order);
+    hipLaunchKernelGGL(psa_order::psa_chunk_sort_kernel, dim3(p.wg_groups), dim3(256), 0, (hipStream_t)stream, cost, (int)total, p.wg_chunk, order);
     if (int e = psa_check_launch("psa_fwd (row order)")) return e;
     p.order = order;
   }
@@ -1001,7 +921,7 @@ extern "C" int psa_fwd_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor
 
 namespace {
 constexpr int64_t FWD_NOALLOC_MAX_ROWS = 1 << 16;  // B * Hq * ceil(L / block_m)
-constexpr size_t FWD_NOALLOC_BYTES = 2 * (size_t)(FWD_NOALLOC_MAX_ROWS + 16 * FWD_MAX_PHASES) * sizeof(int32_t);
+constexpr size_t FWD_NOALLOC_BYTES = 2 * (size_t)(FWD_NOALLOC_MAX_ROWS + 16 * psa_order::MAX_PHASES) * sizeof(int32_t);
 constexpr int FWD_NOALLOC_MAX_DEVICES = 64;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[FWD_NOALLOC_BYTES];

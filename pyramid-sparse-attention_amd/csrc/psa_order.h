@@ -1,0 +1,103 @@
+// Issue order of workgroups: dealing to the XCDs and longest-first sorting (shared by the forward and backward walks).
+//
+// Workgroup ids are dealt round-robin to the 8 XCDs and each XCD runs its ids in order.  The work items (rows of the
+// level map, or kv-block slots of the dK/dV walk) are cut into `groups` contiguous shares of `chunk` items, share g
+// runs on XCD g % 8, the shares of an XCD one after the other: items that are neighbours (same head, so the same
+// K/V or Q/dO) meet in one XCD's L2, and only a few heads are in flight at a time.  Inside a share the items are
+// issued by decreasing cost, which shortens the tail of the launch.  The order only changes WHEN an item is
+// computed, never its result.
+#pragma once
+#include "psa_common.h"
+
+namespace psa_order {
+namespace {  // one private copy per translation unit that launches them
+
+constexpr int COST_BINS = 2048;
+constexpr int MAX_PHASES = 64;
+constexpr int64_t PHASE_BYTES = 128ll << 20;  // operand bytes (K/V + pooled levels, or Q/dO) in use at one time
+
+// position in the dealt order of workgroup `bid` (chunk items per share): share ((bid >> 3) / chunk) * 8 + (bid & 7)
+__device__ __forceinline__ int dealt_entry(int bid, int chunk) {
+  return (((bid >> 3) / chunk) * 8 + (bid & 7)) * chunk + (bid >> 3) % chunk;
+}
+
+// shares for `total` items whose streamed operands take operand_bytes over n_heads (batch x head) slices
+static inline void deal(int64_t total, double operand_bytes, int n_heads, int& chunk, int& groups) {
+  int phases = (int)(operand_bytes / (double)PHASE_BYTES) + 1;
+  const int max_phases = n_heads < MAX_PHASES ? n_heads : MAX_PHASES;
+  phases = phases > max_phases ? max_phases : phases;
+  groups = 8 * phases;
+  chunk = (int)((total + groups - 1) / groups);
+}
+
+// tiles of 64 (pooled) keys that each row of the level map retains: the cost of a row walk
+__global__ __launch_bounds__(256) void psa_row_cost_kernel(const void* map, int map_elem, int total, int Mq, int Nk, int bn_log2,
+                                                         int bm, int causal, int32_t* cost) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= total) return;
+  const int I = row % Mq;
+  int jmax = Nk;
+  if (causal) {
+    const int ce = (int)((((int64_t)(I + 1) * bm) + (1 << bn_log2) - 1) >> bn_log2);
+    jmax = ce < jmax ? ce : jmax;
+  }
+  int cnt[4] = {0, 0, 0, 0};
+  for (int j0 = 0; j0 < jmax; j0 += 64) {
+    const int j = j0 + lane;
+    const int lvl = j < jmax ? load_map(map, (int64_t)row * Nk + j, map_elem) : 0;
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) cnt[lv] += __popcll(__ballot(lvl == (1 << lv)));
+  }
+  if (lane == 0) {
+    int tiles = 0;
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) tiles += ((cnt[lv] << (bn_log2 - lv)) + 63) >> 6;
+    cost[row] = tiles < COST_BINS - 1 ? tiles : COST_BINS - 1;
+  }
+}
+
+// one workgroup per share: counting sort of its items by decreasing cost (order[] holds item ids, -1 past the last item)
+__global__ __launch_bounds__(256) void psa_chunk_sort_kernel(const int32_t* cost, int total, int chunk, int32_t* order) {
+  __shared__ int hist[COST_BINS];
+  const int x = blockIdx.x, tid = threadIdx.x;
+  const int r0 = x * chunk;
+  for (int i = tid; i < COST_BINS; i += 256) hist[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < chunk; i += 256)
+    if (r0 + i < total) atomicAdd(&hist[cost[r0 + i]], 1);
+  __syncthreads();
+  {  // start offset of every bin, highest cost first: thread i owns the 8 bins COST_BINS-1-8i .. COST_BINS-8-8i
+    __shared__ int part[256];
+    constexpr int PER = COST_BINS / 256;
+    int c[PER], sum = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      c[j] = hist[COST_BINS - 1 - (tid * PER + j)];
+      sum += c[j];
+    }
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {  // inclusive scan over the threads
+      const int add = tid >= d ? part[tid - d] : 0;
+      __syncthreads();
+      part[tid] += add;
+      __syncthreads();
+    }
+    int run = part[tid] - sum;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      hist[COST_BINS - 1 - (tid * PER + j)] = run;
+      run += c[j];
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < chunk; i += 256) {
+    if (r0 + i < total) order[r0 + atomicAdd(&hist[cost[r0 + i]], 1)] = r0 + i;
+  }
+  // ids past the last row of the last share
+  const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;
+  for (int i = valid + tid; i < chunk; i += 256) order[r0 + i] = -1;
+}
+
+}  // namespace
+}  // namespace psa_order
