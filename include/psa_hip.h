@@ -40,7 +40,9 @@ extern "C" {
 
 typedef void* psa_stream_t; /* hipStream_t */
 
-/* [B, H, L, D] bf16 view; strides in elements; the D stride is 1. */
+/* [B, H, L, D] bf16 view; strides in elements; the D stride is 1.  Every entry point computes on bf16 operands with
+ * fp32 accumulation and takes bf16 tensors only: a caller that holds fp16 / fp32 tensors (the reference accepts them)
+ * rounds them to bf16 first, as the Python mirror does, and the results then carry that input rounding. */
 typedef struct psa_tensor4 {
   void* ptr;
   int64_t stride_b;
