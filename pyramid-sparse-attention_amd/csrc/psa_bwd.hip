@@ -606,6 +606,76 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
   }
 
+  // ---- 128-key level-0 slot: this workgroup owns 128 tokens of dK / dV outright.  The pooled levels' launch has
+  // finished, so the tokens' shares of the pooled gradients (1/l of pooled row n >> level; for the last real token
+  // also those of the replicate-pad tokens behind it) are added here and dK, dV leave as bf16: no fp32 level-0
+  // buffer, no separate pass.  Same sums in the same order as psa_bwd_unpool_kernel.
+  if constexpr (WIDE) {
+    const int64_t n = key_row0 + key_local;
+    if (n < L) {
+      const int64_t BH = (int64_t)p.B * p.Hkv, npad = p.npad;
+      const float* lk[3];
+      const float* lvv[3];
+#pragma unroll
+      for (int l = 1; l < 4; ++l) {
+        const int64_t rows = BH * npad + pool_row_offset(l, BH, bhk, npad);
+        lk[l - 1] = p.wk + rows * D;
+        lvv[l - 1] = p.wv + rows * D;
+      }
+      bf16_t* dkp = p.dk + b * p.dk_sb + hk * p.dk_sh + n * p.dk_sl;
+      bf16_t* dvp = p.dv + b * p.dv_sb + hk * p.dv_sh + n * p.dv_sl;
+      const float scale = p.scale;
+      auto contrib = [&](const float* const (&w)[3], int64_t row, int col) __attribute__((always_inline)) {
+        f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int l = 1; l < 4; ++l) {
+          const f32x4 x = *(const f32x4*)(w[l - 1] + (row >> l) * D + col);
+          const float inv = 1.0f / (float)(1 << l);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[e] += x[e] * inv;
+        }
+        return a;
+      };
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int col = db * 32 + g * 8 + hh * 4;
+          f32x4 gk, gv;
+#pragma unroll
+          for (int e2 = 0; e2 < 4; ++e2) {
+            gk[e2] = dk[db][g * 4 + e2] * scale;
+            gv[e2] = dv[db][g * 4 + e2];
+          }
+          {
+            const f32x4 ak = contrib(lk, n, col), av = contrib(lvv, n, col);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              gk[e] += ak[e];
+              gv[e] += av[e];
+            }
+          }
+          if (n == L - 1) {  // gradient of the replicate-pad rows lands on the last real token
+            for (int64_t r = L; r < npad; ++r) {
+              const f32x4 ak = contrib(lk, r, col), av = contrib(lvv, r, col);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                gk[e] += ak[e];
+                gv[e] += av[e];
+              }
+            }
+          }
+          u32x2 ok_, ov_;
+          ok_[0] = pack_bf16x2(gk[0], gk[1]);
+          ok_[1] = pack_bf16x2(gk[2], gk[3]);
+          ov_[0] = pack_bf16x2(gv[0], gv[1]);
+          ov_[1] = pack_bf16x2(gv[2], gv[3]);
+          *(u32x2*)(dkp + col) = ok_;
+          *(u32x2*)(dvp + col) = ov_;
+        }
+    }
+    return;
+  }
   // ---- combine the two query halves (<= 64 keys) and write this workgroup's rows of the level buffers ----
   __syncthreads();
   float* red = (float*)smem;  // [2 key halves][2 tensors][DB*16][64 lanes]
@@ -841,7 +911,17 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       hipLaunchKernelGGL(kern, dim3((unsigned)(chunk * groups)), dim3(256), shmem, st, p, slot_lo, slot_cnt, (int)n_wg, chunk, order);
       return PSA_OK;
     };
-    int rl = PSA_OK;
+    // the pooled levels first: the 128-key level-0 launch adds their rows to its own and writes dK, dV
+    const int lo = wide0 ? 1 : 0;
+    int rl;
+    if (causal)
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
+    else
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
+    PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
+    if (int e = psa_check_launch("psa_bwd (dK/dV)")) return e;
     if (wide0) {
       if (causal)
         rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
@@ -850,20 +930,10 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
         rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
                       : launch(psa_bwd_dkdv_lds_kernel<64, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
       PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
-      if (int e = psa_check_launch("psa_bwd (dK/dV, 128-key slots)")) return e;
+      return psa_check_launch("psa_bwd (dK/dV, 128-key slots)");
     }
-    const int lo = wide0 ? 1 : 0;
-    if (causal)
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
-    else
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
-    PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
-    const int rc = psa_check_launch("psa_bwd (dK/dV)");
-    if (rc != PSA_OK) return rc;
   }
-  // 4. un-pool
+  // 4. un-pool (blocks of 64 or 32 keys: every level went to the fp32 buffers)
   {
     const int64_t units = (int64_t)L * (D / 4);
     dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * Hkv), 2);
