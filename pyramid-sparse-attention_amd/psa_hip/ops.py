@@ -439,6 +439,9 @@ def sparse_attention_fwd(
 
 
 _SIDE_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
+# below this size of K the fork / join of the second stream costs more than the overlap gains (small layers are bound by
+# launch latency: 0.07 ms against 0.13 ms with the fork at B1 H2 N4096 D64)
+_SIDE_STREAM_MIN_BYTES = 16 << 20
 
 
 def _side_stream(device: torch.device) -> "torch.cuda.Stream":
@@ -470,7 +473,7 @@ def psa_layer_fwd(
     """estimate (+ level map, in the estimator's reduction kernel) -> pooled K/V -> sparse attention, non-causal,
     no gradient, with a dense int8 level map in between (no index-list round trip).  The pooling pass (HBM-bound,
     independent of the estimate) runs on a second stream of default priority beside the estimator and joins the current
-    stream before the attention kernel: worth 0.02 ms of 1.0 at the Wan2.1 shape."""
+    stream before the attention kernel (worth 0.02 ms of 1.0 at the Wan2.1 shape), unless the layer is small."""
     _require_gpu(q, k, v)
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     keep_m, keep_n = block_m // 4, block_n // 4
@@ -480,7 +483,8 @@ def psa_layer_fwd(
         # pass reads K, V through the index and leaves the re-ordered rows behind, the estimator and the attention kernel
         # read Q through it, and the attention kernel writes its rows back to their original places
         kp, vp, kb, vb = pool_kv_indexed(kb, vb, token_index, block_n)
-    else:
+    side = None
+    if token_index is None and kb.numel() * 2 >= _SIDE_STREAM_MIN_BYTES:
         # the buffers come from the current stream's allocator; the side stream only runs the kernel
         main = torch.cuda.current_stream(qb.device)
         side = _side_stream(qb.device)
@@ -494,8 +498,10 @@ def psa_layer_fwd(
                               compute_tile=tile_n, map_dtype=torch.int8, sm_scale=sm_scale, q_index=token_index)
     if level_cap is not None:
         mp = map_min_cap(mp, level_cap)
-    if token_index is None:
+    if side is not None:
         main.wait_stream(side)
+    elif token_index is None:
+        kp, vp = pool_kv(kb, vb, block_n)
     out = sparse_attention_fwd(qb, kb, vb, mp, block_m, block_n, sm_scale, pools=(kp, vp), q_index=token_index)
     if out.dtype != q.dtype:
         out = out.to(q.dtype)
