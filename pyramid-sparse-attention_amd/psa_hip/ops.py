@@ -469,11 +469,16 @@ def psa_layer_fwd(
     return_map: bool = False,
     text_length: int = 0,
     token_index: Optional[torch.Tensor] = None,
+    sim_thresholds: Optional[Tuple[float, float, float]] = None,
+    return_cap: bool = False,
 ):
     """estimate (+ level map, in the estimator's reduction kernel) -> pooled K/V -> sparse attention, non-causal,
     no gradient, with a dense int8 level map in between (no index-list round trip).  The pooling pass (HBM-bound,
     independent of the estimate) runs on a second stream of default priority beside the estimator and joins the current
-    stream before the attention kernel (worth 0.02 ms of 1.0 at the Wan2.1 shape), unless the layer is small."""
+    stream before the attention kernel (worth 0.02 ms of 1.0 at the Wan2.1 shape), unless the layer is small.
+    sim_thresholds (t2, t4, t8): the key-similarity cap is computed here, on the keys in the order the layer works in
+    (after the re-ordering), and applied to the map; level_cap passes a ready cap instead.  Returns out, or
+    (out[, map][, cap]) with return_map / return_cap."""
     _require_gpu(q, k, v)
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
     keep_m, keep_n = block_m // 4, block_n // 4
@@ -494,6 +499,10 @@ def psa_layer_fwd(
         side.wait_stream(main)
         with torch.cuda.stream(side):
             pool_kv(kb, vb, block_n, out=(kp, vp))
+    if sim_thresholds is not None:
+        if level_cap is not None:
+            raise ValueError("pass either level_cap or sim_thresholds")
+        level_cap = k_similarity(kb, block_n, *sim_thresholds)
     mp = estimate_sampled_map(qb, kb, off_q, off_k, block_m, block_n, keep_m, keep_n, mask_ratios, text_length, mode,
                               compute_tile=tile_n, map_dtype=torch.int8, sm_scale=sm_scale, q_index=token_index)
     if level_cap is not None:
@@ -505,7 +514,9 @@ def psa_layer_fwd(
     out = sparse_attention_fwd(qb, kb, vb, mp, block_m, block_n, sm_scale, pools=(kp, vp), q_index=token_index)
     if out.dtype != q.dtype:
         out = out.to(q.dtype)
-    return (out, mp) if return_map else out
+    if not (return_map or return_cap):
+        return out
+    return (out,) + ((mp,) if return_map else ()) + ((level_cap,) if return_cap else ())
 
 
 # ----------------------------------------------------------------------------- attention backward

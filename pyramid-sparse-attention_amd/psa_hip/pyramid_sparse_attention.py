@@ -182,15 +182,13 @@ class PyramidSparseAttention(nn.Module):
             out_r = ops.sparse_attention_fwd(q_r, k_r, v_r, None, 128, 128)  # dense attention, same kernel
             sparsity = 0.0
             per_head_density = [1.0] * q_r.shape[1] if compute_stats else []
+        elif not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
+            out_r, sparsity, per_head_density, sim_cap = self._sparse_layer(q_r, k_r, v_r, fused, compute_stats)
+            if compute_stats:
+                self.sparsity_acc = self.sparsity_acc + sparsity
         else:
-            index = pools = None
-            if fused:
-                index = self.rearranger.token_index(q.device)
-                kp, vp, k_r, v_r = ops.pool_kv_indexed(k, v, index, self.config.block_n)
-                pools = (kp, vp)
             out_r, sparsity, per_head_density, sim_cap = adaptive_block_sparse_attn(
-                q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets,
-                q_index=index, pools=pools
+                q_r, k_r, v_r, self.config, self.sparse_attention_fn, compute_stats=compute_stats, sample_offsets=self.sample_offsets
             )
             if compute_stats:
                 self.sparsity_acc = self.sparsity_acc + sparsity
@@ -201,10 +199,40 @@ class PyramidSparseAttention(nn.Module):
                                      is_warmup=is_warmup)
         return self.rearranger.reversed_rearrange(out_r) if restore else out_r
 
+    def _sparse_layer(self, q, k, v, through_index, compute_stats):
+        """The sparse layer without gradients through the layer operator (ops.psa_layer_fwd): estimate and level map in
+        two launches, the similarity cap, pooling and the token re-ordering inside the layer's kernels, and a dense
+        int8 level map for either mask type (the index-list modes select the same levels and ignore the text
+        columns).  Same outputs, bit for bit, as adaptive_block_sparse_attn on re-ordered tensors."""
+        cfg = self.config
+        B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
+        if self.sample_offsets is None:
+            off_q = draw_sample_offsets(B, H, cfg.block_m, cfg.block_m // 4, q.device)
+            off_k = draw_sample_offsets(B, Hkv, cfg.block_n, cfg.block_n // 4, k.device)
+        else:
+            off_q, off_k = self.sample_offsets
+        if cfg.mask_mode not in ("topk", "thresholdbound"):
+            raise ValueError(f"Unknown mask_mode: {cfg.mask_mode}")
+        thr = None
+        if getattr(cfg, "use_sim_mask", True):
+            thr = (float(cfg.sim_2x_threshold), float(cfg.sim_4x_threshold), float(cfg.sim_8x_threshold))
+        out, mp, cap = ops.psa_layer_fwd(
+            q, k, v, off_q, off_k, cfg.mask_ratios, cfg.mask_mode, cfg.block_m, cfg.block_n, cfg.tile_n,
+            text_length=cfg.text_length if cfg.attn_impl == "old_mask_type" else 0,
+            token_index=self.rearranger.token_index(q.device) if through_index else None,
+            sim_thresholds=thr, return_map=True, return_cap=True)
+        if compute_stats:
+            d = ops.density(mp)  # [B*H + 1] on the device
+            return out, 1 - d[-1], d[:-1].view(B, H).mean(0), cap
+        return out, 0.0, [], cap
+
     def close_logger(self):
         if self.logger is not None:
             self.logger.close()
 
     def __del__(self):
         if getattr(self, "logger", None) is not None:
-            self.logger.close()
+            try:
+                self.logger.close()
+            except Exception:  # the interpreter is shutting down: builtins and torch may already be gone
+                pass
