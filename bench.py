@@ -371,6 +371,24 @@ def main():
                "layer_with_gather_passes": round(t_l2, 4), "outputs_bit_identical": reorder_equal}
     del q0, k0, v0
 
+    # ---- the same layer through the module API with what the reference's preset for this model turns on (Gilbert
+    # re-ordering, key-similarity cap; similarity thresholds of the preset); inputs in raster order
+    preset = None
+    if args.workload == "c2":
+        from psa_hip.pyramid_sparse_attention import AttentionConfig, PyramidSparseAttention
+
+        cfg = AttentionConfig(width=gw, height=gh, depth=gd, text_length=text, use_rearrange=True, rearrange_method="Gilbert",
+                              attn_impl="old_mask_type", mask_mode=mode, warmup_steps=0, use_sim_mask=True, block_m=bm, block_n=bn,
+                              tile_n=tn, mask_ratios=ratios, sim_2x_threshold=0.7, sim_4x_threshold=0.65, sim_8x_threshold=0.6,
+                              enable_logging=False)
+        mod = PyramidSparseAttention(cfg, inference_num=50, layer_num=30, model_type="wan")
+        mod.sample_offsets = (off_q, off_k)
+        with torch.inference_mode():
+            t_mod, _ = time_gpu(lambda: mod(q, k, v, 0), it)
+            t_ks, _ = time_gpu(lambda: ops.k_similarity(k, bn, 0.7, 0.65, 0.6), it)
+        preset = {"module_layer": round(t_mod, 4), "k_similarity": round(t_ks, 4),
+                  "what": "PyramidSparseAttention.forward, Gilbert re-ordering through the token index + similarity cap"}
+
     # ---- what the chip sustains on a register-only MFMA loop, measured now (constant and random operands) ----
     _l = probe_lib()
 
@@ -492,6 +510,7 @@ def main():
         "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
                       "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4)},
         "reorder_ms": reorder,
+        "preset_ms": preset,
         "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),
         "pct_bf16_peak_fwd_executed": round(100 * exec_flops / (t_fwd_med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
         "pool_gbs": round(pool_bytes / (t_pool * 1e-3) / 1e9, 1),
