@@ -239,7 +239,8 @@ int psa_fwd_noalloc(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
                     int causal, psa_stream_t stream);
 int64_t psa_fwd_noalloc_max_rows(void);
 
-/* Bytes of workspace psa_bwd needs (fp32 dK/dV per pyramid level, delta, lse in log2 units). */
+/* Bytes of workspace psa_bwd needs (fp32 dK/dV per pyramid level, delta, lse in log2 units, cost and issue order of
+ * the dQ rows and of the dK/dV workgroups). */
 int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n);
 
 /* Backward of psa_fwd w.r.t. q, k, v (the map carries no gradient).  dq/dk/dv are bf16 views like
