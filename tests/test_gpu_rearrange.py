@@ -158,3 +158,36 @@ def test_module_reordering_without_gather_passes(impl, mode, blocks, monkeypatch
     got = run(True)
     assert (got[0].float() - ref[0].float()).abs().max().item() <= 2e-2
     assert torch.equal(got[1], ref[1]) and torch.equal(got[2], ref[2])
+
+
+@pytest.mark.parametrize("impl,mode,blocks,sim", [("new_mask_type", "topk", (64, 64, 32), False),
+                                                  ("old_mask_type", "thresholdbound", (128, 128, 32), True),
+                                                  ("old_mask_type", "topk", (128, 128, 32), True)])
+def test_module_layer_operator_equals_stage_by_stage(impl, mode, blocks, sim):
+    """Without gradients PyramidSparseAttention runs its sparse layer through the layer operator (fused estimate + map,
+    similarity cap, token index).  The result must be the same bits as the reference's sequence of separate stages
+    (estimate -> transfer_attn_to_mask -> min with the similarity cap -> sparse attention) on gathered tensors."""
+    from psa_hip.pyramid_sparse_attention import AttentionConfig, PyramidSparseAttention, adaptive_block_sparse_attn
+    from psa_hip.utils.synthetic import sample_offsets
+
+    depth, height, width, text = 3, 10, 24, 40
+    L = depth * height * width + text
+    cfg = AttentionConfig(width=width, height=height, depth=depth, text_length=text, use_rearrange=True, rearrange_method="Gilbert",
+                          attn_impl=impl, mask_mode=mode, warmup_steps=0, use_sim_mask=sim, block_m=blocks[0], block_n=blocks[1],
+                          tile_n=blocks[2], sim_2x_threshold=0.3, sim_4x_threshold=0.2, sim_8x_threshold=0.1, enable_logging=False,
+                          mask_ratios={1: (0.0, 0.4), 2: (0.4, 0.6), 4: (0.6, 0.8), 8: (0.8, 0.9), 0: (0.9, 1.0)})
+    g = torch.Generator(device="cpu").manual_seed(11)
+    base = torch.randn(1, 4, 1, 128, generator=g)
+    q, k, v = ((base + 0.7 * torch.randn(1, 4, L, 128, generator=g)).to(torch.bfloat16).to(dev()) for _ in range(3))
+    offs = (sample_offsets(1, 4, cfg.block_m, cfg.block_m // 4, 1, device=dev()),
+            sample_offsets(1, 4, cfg.block_n, cfg.block_n // 4, 2, device=dev()))
+    m = PyramidSparseAttention(cfg, inference_num=4, layer_num=1, model_type="cogvideo")
+    m.sample_offsets = offs
+    with torch.no_grad():
+        got = m(q, k, v, 0)
+        q_r, k_r, v_r = m.rearranger.rearrange(q, k, v)
+        out_r, _, _, cap = adaptive_block_sparse_attn(q_r, k_r, v_r, cfg, m.sparse_attention_fn, sample_offsets=offs)
+        ref = m.rearranger.reversed_rearrange(out_r)
+    assert torch.equal(got, ref)
+    if sim:
+        assert cap is not None and int((cap > 1).sum()) > 0  # the cap really acts in this case
