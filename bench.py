@@ -245,6 +245,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention comparison legs (keeps kernel profiles clean)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the token re-ordering and preset legs (reorder_ms, preset_ms): a profile then holds the timed layer's "
+                         "kernels only")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--copy-calib", action="store_true",
                     help="after the run, stream 1 GiB through a plain elementwise kernel (reads 1 GiB, writes 1 GiB): "
@@ -343,51 +346,52 @@ def main():
         t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
         t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
 
-    # ---- token re-ordering: the layer on tokens already in curve order (above), the same layer reading / writing through
-    # the token index (no gather passes), and with explicit gather passes before and after; the inputs of the last two
-    # are the un-gathered q, k, v, so all three compute the same layer and the outputs must agree bit for bit
-    from psa_hip.utils.rearranger import GilbertRearranger
+    reorder = preset = None
+    if not args.no_extras:
+        # ---- token re-ordering: the layer on tokens already in curve order (above), the same layer reading / writing through
+        # the token index (no gather passes), and with explicit gather passes before and after; the inputs of the last two
+        # are the un-gathered q, k, v, so all three compute the same layer and the outputs must agree bit for bit
+        from psa_hip.utils.rearranger import GilbertRearranger
 
-    gd, gh, gw = w["grid"]
-    rr = GilbertRearranger(gw, gh, gd, text)
-    idx = rr.token_index(dev)
-    inv = rr._combined_index(dev, False)
-    q0, k0, v0 = ops.gather_rows((q, k, v), inv)  # q0[idx[i]] = q[i]
+        gd, gh, gw = w["grid"]
+        rr = GilbertRearranger(gw, gh, gd, text)
+        idx = rr.token_index(dev)
+        inv = rr._combined_index(dev, False)
+        q0, k0, v0 = ops.gather_rows((q, k, v), inv)  # q0[idx[i]] = q[i]
 
-    def layer_indexed():
-        return ops.psa_layer_fwd(q0, k0, v0, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text, token_index=idx)
+        def layer_indexed():
+            return ops.psa_layer_fwd(q0, k0, v0, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text, token_index=idx)
 
-    def layer_gathered():
-        qg, kg, vg = ops.gather_rows((q0, k0, v0), idx)
-        og = ops.psa_layer_fwd(qg, kg, vg, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text)
-        return ops.gather_rows((og,), inv)[0]
+        def layer_gathered():
+            qg, kg, vg = ops.gather_rows((q0, k0, v0), idx)
+            og = ops.psa_layer_fwd(qg, kg, vg, off_q, off_k, ratios, mode, bm, bn, tn, text_length=text)
+            return ops.gather_rows((og,), inv)[0]
 
-    o_ref = layer()
-    reorder_equal = bool(torch.equal(layer_indexed(), layer_gathered())) and bool(torch.equal(ops.gather_rows((layer_indexed(),), idx)[0], o_ref))
-    t_l0, _ = time_gpu(layer, it)
-    t_l1, _ = time_gpu(layer_indexed, it)
-    t_l2, _ = time_gpu(layer_gathered, it)
-    reorder = {"layer_tokens_already_ordered": round(t_l0, 4), "layer_through_token_index": round(t_l1, 4),
-               "layer_with_gather_passes": round(t_l2, 4), "outputs_bit_identical": reorder_equal}
-    del q0, k0, v0
+        o_ref = layer()
+        reorder_equal = bool(torch.equal(layer_indexed(), layer_gathered())) and bool(torch.equal(ops.gather_rows((layer_indexed(),), idx)[0], o_ref))
+        t_l0, _ = time_gpu(layer, it)
+        t_l1, _ = time_gpu(layer_indexed, it)
+        t_l2, _ = time_gpu(layer_gathered, it)
+        reorder = {"layer_tokens_already_ordered": round(t_l0, 4), "layer_through_token_index": round(t_l1, 4),
+                   "layer_with_gather_passes": round(t_l2, 4), "outputs_bit_identical": reorder_equal}
+        del q0, k0, v0
 
-    # ---- the same layer through the module API with what the reference's preset for this model turns on (Gilbert
-    # re-ordering, key-similarity cap; similarity thresholds of the preset); inputs in raster order
-    preset = None
-    if args.workload == "c2":
-        from psa_hip.pyramid_sparse_attention import AttentionConfig, PyramidSparseAttention
+        # ---- the same layer through the module API with what the reference's preset for this model turns on (Gilbert
+        # re-ordering, key-similarity cap; similarity thresholds of the preset); inputs in raster order
+        if args.workload == "c2":
+            from psa_hip.pyramid_sparse_attention import AttentionConfig, PyramidSparseAttention
 
-        cfg = AttentionConfig(width=gw, height=gh, depth=gd, text_length=text, use_rearrange=True, rearrange_method="Gilbert",
-                              attn_impl="old_mask_type", mask_mode=mode, warmup_steps=0, use_sim_mask=True, block_m=bm, block_n=bn,
-                              tile_n=tn, mask_ratios=ratios, sim_2x_threshold=0.7, sim_4x_threshold=0.65, sim_8x_threshold=0.6,
-                              enable_logging=False)
-        mod = PyramidSparseAttention(cfg, inference_num=50, layer_num=30, model_type="wan")
-        mod.sample_offsets = (off_q, off_k)
-        with torch.inference_mode():
-            t_mod, _ = time_gpu(lambda: mod(q, k, v, 0), it)
-            t_ks, _ = time_gpu(lambda: ops.k_similarity(k, bn, 0.7, 0.65, 0.6), it)
-        preset = {"module_layer": round(t_mod, 4), "k_similarity": round(t_ks, 4),
-                  "what": "PyramidSparseAttention.forward, Gilbert re-ordering through the token index + similarity cap"}
+            cfg = AttentionConfig(width=gw, height=gh, depth=gd, text_length=text, use_rearrange=True, rearrange_method="Gilbert",
+                                  attn_impl="old_mask_type", mask_mode=mode, warmup_steps=0, use_sim_mask=True, block_m=bm, block_n=bn,
+                                  tile_n=tn, mask_ratios=ratios, sim_2x_threshold=0.7, sim_4x_threshold=0.65, sim_8x_threshold=0.6,
+                                  enable_logging=False)
+            mod = PyramidSparseAttention(cfg, inference_num=50, layer_num=30, model_type="wan")
+            mod.sample_offsets = (off_q, off_k)
+            with torch.inference_mode():
+                t_mod, _ = time_gpu(lambda: mod(q, k, v, 0), it)
+                t_ks, _ = time_gpu(lambda: ops.k_similarity(k, bn, 0.7, 0.65, 0.6), it)
+            preset = {"module_layer": round(t_mod, 4), "k_similarity": round(t_ks, 4),
+                      "what": "PyramidSparseAttention.forward, Gilbert re-ordering through the token index + similarity cap"}
 
     # ---- what the chip sustains on a register-only MFMA loop, measured now (constant and random operands) ----
     _l = probe_lib()
