@@ -225,6 +225,30 @@ int psa_fwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, con
  * (src/psa_triton/kernels/psa_kernel.py:398-431). */
 int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m);
 
+/* Tile schedule of a level map: what the attention kernel walks, built once per map instead of inside every launch
+ * that walks it.  Per (batch, head, q-block) row it holds the row's tiles of 64 pooled keys (level, source rows, fill,
+ * diagonal / ragged flags: 16 bytes per tile) and the rows' issue order (dealt to the chip's XCDs, longest first, equal
+ * rows in index order - the same order in every run).  It is the counterpart of the reference's index list, which is
+ * also computed once per map and then walked by the kernel:
+ *   reference src/psa_triton/utils/transfer_attn_to_mask.py:271-500 (list built), src/psa_triton/kernels/psa_kernel.py:207-302 (walked).
+ * Schedules exist for D = 128, block_m = block_n = 128 (psa_schedule_bytes returns 0 otherwise and psa_build_schedule
+ * PSA_ERR_UNSUPPORTED; psa_fwd covers every shape).  `schedule`: caller-allocated device memory of psa_schedule_bytes(...)
+ * bytes, 16-byte aligned (the bound is the worst case, every pair at level 1: 32 bytes per (q-block, kv-block) pair; only
+ * the retained tiles are written and read).  It stays valid for as long as the map is unchanged and may be used by any
+ * number of psa_fwd_scheduled calls with the same shape arguments. */
+int64_t psa_schedule_bytes(int B, int Hq, int Hkv, int L, int D, int block_m, int block_n);
+int psa_build_schedule(const void* map, int map_elem_bytes, void* schedule, int B, int Hq, int Hkv, int L, int D,
+                       int block_m, int block_n, int causal, psa_stream_t stream);
+
+/* psa_fwd on a prebuilt schedule (same results as psa_fwd on the map the schedule was built from; rows are walked in
+ * the same tile order).  q_index may be NULL; otherwise as in psa_fwd_indexed.  `map` is the map the schedule was built
+ * from (kept in the signature for the shapes' sake; the kernel reads the schedule).
+ * Replaces the same reference code as psa_fwd. */
+int psa_fwd_scheduled(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
+                      const void* v_pool, const void* map, int map_elem_bytes, const void* schedule, psa_tensor4 out,
+                      float* lse, int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
+                      int causal, psa_stream_t stream);
+
 /* psa_fwd without a workspace argument and without any allocation: the row-ordering scratch is a fixed array inside
  * the library (one copy per GPU, about 0.5 MiB, held until the process ends).  This entry point has no counterpart in
  * the reference; it exists for callers that cannot allocate device memory around the call - code under HIP graph

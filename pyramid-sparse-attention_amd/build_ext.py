@@ -19,6 +19,9 @@ FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-Wno-unused-command-line-argument",
+    # the tile-copy helpers write M0 in inline assembly and say so in their clobber lists (the compiler must not assume
+    # that a value it left in M0 survives them); M0 being a reserved register, every such list draws a warning
+    "-Wno-inline-asm",
     # no packed fp32 arithmetic in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
@@ -66,22 +69,7 @@ def build(verbose=True, extra_flags=(), out=OUT):
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
     if verbose:
         print("built", out)
-    if out == OUT:
-        build_probe(verbose)
     return out
-
-
-PROBE_SRC = os.path.join(HERE, "bench_probe", "psa_probe.hip")
-PROBE_OUT = os.path.join(HERE, "bench_probe", "libpsa_probe.so")
-
-
-def build_probe(verbose=True):
-    """bench.py's optional helper (synthetic MFMA / attention-shaped loops): a library of its own, outside the C ABI.
-    Compiled like the forward kernel it models."""
-    _run([_hipcc(), *FLAGS, "-fno-honor-nans", "-shared", "-o", PROBE_OUT, PROBE_SRC])
-    if verbose:
-        print("built", PROBE_OUT)
-    return PROBE_OUT
 
 
 if __name__ == "__main__":

@@ -34,6 +34,7 @@
 #include "psa_common.h"
 #include "psa_tiles.h"
 #include "psa_order.h"
+#include "psa_schedule.h"
 
 namespace {
 
@@ -72,6 +73,10 @@ struct FwdParams {
   int grp_bytes;  // two-group kernel: LDS bytes of one group (tile buffers + schedule)
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
   const int32_t* q_index;  // optional (token re-ordering): query / output position i lives in row q_index[i] of q, out, lse
+  // prebuilt tile schedule (psa_schedule.h), scheduled kernel only: tiles per row and the rows' tile records
+  const u32x4* sched_rec;
+  const int32_t* sched_tiles;
+  int rec_stride;
 };
 
 constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the blocks of a tile
@@ -377,7 +382,14 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
 // exponentials.
 #define PP_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-template <int D, int NW>
+// GS: the rows' tiles come from a prebuilt schedule in device memory (psa_schedule.h; 128-key blocks, K / V rows D
+// elements apart) instead of being compacted from the map row here.  A wave fetches ONE word per tile (a scalar load,
+// three tiles ahead): level, fill and the first source row of the 16-row quarter it copies.  A wave issues at most one
+// instruction per 4 cycles whatever its kind, so what bounds the vector phase is its instruction COUNT: a copy here is
+// two instructions (M0, then the load with the row step n * 256 as its immediate offset - which the hardware also adds
+// on the LDS side, so M0 carries the difference), the base pointer of a tile's level is kept while the level stays the
+// same (tiles of a row are sorted by level), and nothing is looked up per lane.
+template <int D, int NW, bool GS>
 __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p) {
   using G = psa_tiles::LtGeom<D>;
   constexpr int F_TILE = G::TILE;
@@ -409,6 +421,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   const int bid = blockIdx.x, sc = p.wg_chunk >> 1;
   const int entry = ((((bid >> 3) / sc) * 8 + (bid & 7)) * sc + (bid >> 3) % sc) * 2 + grp;
   int logical = p.order != nullptr ? p.order[entry] : entry;
+  logical = __builtin_amdgcn_readfirstlane(logical);
   const bool active = logical >= 0 && logical < p.total_wg;
   if (!active) logical = 0;
   const int I = logical % p.Mq;
@@ -432,10 +445,20 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
   }
-  // both groups run the builder's barriers together
-  const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2, P_L,
-                                                 P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt[grp], s_ioff[grp], s_toff[grp],
-                                                 s_wcnt[grp], tid);
+  // the row's tile records (GS): read through the scalar cache; wp walks this wave's word of the records
+  using w_ptr = const __attribute__((address_space(4))) uint32_t*;
+  using rec_ptr = const __attribute__((address_space(4))) u32x4*;
+  rec_ptr recs = nullptr;
+  int T;
+  if constexpr (GS) {
+    recs = (rec_ptr)(uintptr_t)(p.sched_rec + (int64_t)logical * p.rec_stride);
+    T = active ? __builtin_amdgcn_readfirstlane(p.sched_tiles[logical]) : 0;
+  } else {
+    // both groups run the builder's barriers together
+    T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2, P_L,
+                                          P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt[grp], s_ioff[grp], s_toff[grp],
+                                          s_wcnt[grp], tid);
+  }
   if (tid == 0) s_T[grp] = T;
 
   const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
@@ -473,7 +496,29 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   // ---- softmax of tile t, in pieces --------------------------------------------------------------------
   // mask_tile: partly filled tiles and the causal diagonal (rare).  head_piece(i): piece i of the row maximum /
   // reference update, small enough to ride along with one MFMA of PV(t-1).  prob16: the exponentials.
-  uint32_t d_cur = 0;  // descriptor word 0 of the tile whose logits are in s
+  uint32_t d_cur = 0;  // descriptor word 0 of the tile whose logits are in s: level | masked << 2 | ...
+  uint32_t w_cur = 0;  // GS: this wave's word of its record
+  auto mask_tile_rec = [&](int t, f32x16 (&s_cur)[2]) __attribute__((always_inline)) {
+    const int lv = psa_sched::rec_level(w_cur);
+    const int nvalid = psa_sched::rec_nvalid(w_cur);
+    const int qlim = (q_idx + 1) >> lv;
+    u32x4 r4 = {0u, 0u, 0u, 0u};
+    if (P_causal) r4 = recs[t];  // the source rows of all four quarters (rare path: fetched on demand)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int r0 = c * 32 + g * 8 + hh * 4;
+        int keep = nvalid - r0;
+        if (P_causal) {
+          // slots r0 .. r0+3 lie in quarter 2c + g/2 of the tile, whose source rows are consecutive
+          const int src0 = psa_sched::rec_src(r4[c * 2 + (g >> 1)]) + (g & 1) * 8 + hh * 4;
+          keep = keep < qlim - src0 ? keep : qlim - src0;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s_cur[c][g * 4 + e] = e < keep ? s_cur[c][g * 4 + e] : -INFINITY;
+      }
+  };
   auto mask_tile = [&](int t, f32x16 (&s_cur)[2]) __attribute__((always_inline)) {
     const uint32_t d = d_cur;
     const int lv = d & 3;
@@ -529,14 +574,18 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   };
   // probabilities of 4 logits: exp2, round to bf16 for P^T; the row sum adds the unrounded values with plain adds
   // (a dot-product instruction would queue behind the other group's MFMAs)
-  auto prob4 = [&](const f32x16& sc, int i, float nb_, uint32_t* pk2, float& lsum) __attribute__((always_inline)) {
+  // (x0: scale * sc[i] + nb_, where the caller already has it - it rides along with a copy in the scheduled walk)
+  auto prob4x = [&](const f32x16& sc, int i, float nb_, uint32_t* pk2, float& lsum, float x0) __attribute__((always_inline)) {
 #pragma unroll
     for (int e = 0; e < 4; e += 2) {
-      const float p0 = fast_exp2(__builtin_fmaf(sc[i + e], P_scale_log2, nb_));
+      const float p0 = fast_exp2(e == 0 ? x0 : __builtin_fmaf(sc[i + e], P_scale_log2, nb_));
       const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb_));
       pk2[e >> 1] = pack_bf16x2(p0, p1);
       lsum += p0 + p1;
     }
+  };
+  auto prob4 = [&](const f32x16& sc, int i, float nb_, uint32_t* pk2, float& lsum) __attribute__((always_inline)) {
+    prob4x(sc, i, nb_, pk2, lsum, __builtin_fmaf(sc[i], P_scale_log2, nb_));
   };
   // Copy source of a tile for this lane: base pointers and row strides of its level (uniform), and the RPL
   // consecutive source rows of this wave's 16-row group (clamped where a partly filled tile runs past the end).
@@ -643,8 +692,66 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
 #pragma unroll
     for (int n = 0; n < G::RPL; ++n) c.row[n] = a.src0[0] + n < a.lim ? a.src0[0] + n : a.lim;
   };
+  // ---- GS: copies addressed from scalar registers ------------------------------------------------------------
+  // A lane fetches rows 4 * (lane / 16) + n of its wave's quarter, n = 0..3; all rows are D * 2 bytes apart.
+  const int lane_row = psa_tiles::lt_fetch_row<D>(lane);
+  const uint32_t voff_s = (uint32_t)lane_row * (uint32_t)(D * 2) + f_chunk;
+  struct Stream {  // where one tensor's tiles currently come from: a level's rows (the level changes 3 times per row)
+    const char* base;
+    uint32_t code;
+  };
+  Stream st_k = {kb0, 0u}, st_v = {vb0, 0u};
+  // first source row of this wave's quarter of the tile with word w; rag: the tile is ragged (rows are clamped per lane)
+  auto quarter_src = [&](Stream& st, bool is_k, uint32_t w, bool& rag) __attribute__((always_inline)) {
+    const uint32_t code = psa_sched::rec_code(w);
+    if (code != st.code) {
+      st.code = code & 3u;  // (a ragged tile comes back here for every tile)
+      st.base = is_k ? by_level((int)(code & 3u), kb0, kb1, kb2, kb3) : by_level((int)(code & 3u), vb0, vb1, vb2, vb3);
+      rag = rag || code == psa_sched::REC_CODE_RAGGED;
+    }
+    return st.base + (uint64_t)((w & psa_sched::REC_SRC_MASK) * (uint32_t)(D * 2));
+  };
+  // copy instruction N of the wave's quarter (tile rows 4i + N of the quarter) into the tile buffer at LDS_BYTE
+  auto issue_s = [&](const char* src, auto lds_byte, auto n) __attribute__((always_inline)) {
+    constexpr int N = decltype(n)::value;
+    psa_tiles::lds_copy16_imm<decltype(lds_byte)::value + N * F_ISTR, N * D * 2>(src, voff_s, wave_lds);
+  };
+  // the same with the first multiply-add of the exponentials that follow in the wait state between the write of M0 and
+  // the copy (returns scale * x + y)
+  auto issue_s_fma = [&](const char* src, auto lds_byte, auto n, float x, float y) __attribute__((always_inline)) {
+    constexpr int N = decltype(n)::value;
+    return psa_tiles::lds_copy16_imm_fma<decltype(lds_byte)::value + N * F_ISTR, N * D * 2>(src, voff_s, wave_lds, P_scale_log2, x, y);
+  };
+  // the same with a row index per lane, clamped to the last token (ragged tiles: the walk takes this form only in
+  // phases that copy such a tile, so that the usual phase has no branch between its copies)
+  auto issue_clamped = [&](const char* base0, uint32_t w, auto lds_byte, auto n) __attribute__((always_inline)) {
+    constexpr int N = decltype(n)::value, OFF = decltype(lds_byte)::value + N * F_ISTR;
+    const int lim = psa_sched::rec_code(w) == psa_sched::REC_CODE_RAGGED ? P_L - 1 : 0x7fffffff;
+    const int row = psa_sched::rec_src(w) + lane_row + N;
+    psa_tiles::lds_copy16_row<OFF>(base0, (uint32_t)(row < lim ? row : lim), (uint32_t)(D * 2), f_chunk, wave_lds);
+  };
+  auto issue_tile = [&](Stream& st, bool is_k, uint32_t w, auto lds_byte) __attribute__((always_inline)) {
+    bool rag = false;
+    const char* src = quarter_src(st, is_k, w, rag);
+    if (rag) static_for<G::RPL>([&](auto n) __attribute__((always_inline)) { issue_clamped(st.base, w, lds_byte, n); });
+    else static_for<G::RPL>([&](auto n) __attribute__((always_inline)) { issue_s(src, lds_byte, n); });
+  };
+  w_ptr wp = nullptr;                    // this wave's word of the record fetched next
+  uint32_t w_v = 0, w_k = 0, w_next = 0;  // words of tiles t+1 (its V goes out next), t+2 (its K), of the next M phase
+  const int T_last = T > 0 ? T - 1 : 0;
   // first copies: K(0), V(0), K(1); ts is left describing tile min(1, T-1) for the copy of V(1)
-  if (T > 0) {
+  if constexpr (GS) {
+    if (T > 0) {
+      wp = (w_ptr)(uintptr_t)((const uint32_t*)(p.sched_rec + (int64_t)logical * p.rec_stride) + wave);
+      w_next = wp[0];  // (records T .. T+2 repeat record T-1)
+      w_v = wp[4];
+      w_k = wp[8];
+      wp += 12;
+      issue_tile(st_k, true, w_next, IC<0>{});
+      issue_tile(st_v, false, w_next, IC<2 * F_TILE>{});
+      if (T > 1) issue_tile(st_k, true, w_v, IC<F_TILE>{});
+    }
+  } else if (T > 0) {
     TileSrc a;
     tile_src(0, a);
     issue_rows(a.kbase, a.kstr, a.lim, a.src0, 0);
@@ -678,16 +785,24 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   // Both phases are free of branches (tiles past the end are clamped to the last one and copied again into a
   // buffer nobody reads), so that the instruction order below is the order that runs.
   constexpr int HOOK0 = 2;  // first PV step that carries a piece of the maximum (QK's last results need that long)
-  const int T_last = T > 0 ? T - 1 : 0;
-  uint32_t d_next = T > 0 ? __builtin_amdgcn_readfirstlane(tdesc[0][0]) : 0u;  // descriptor of the tile of the next M phase
+  uint32_t d_next = 0u;  // descriptor of the tile of the next M phase
+  if constexpr (!GS) d_next = T > 0 ? __builtin_amdgcn_readfirstlane(tdesc[0][0]) : 0u;
   auto mfma_phase = [&](int t, auto cur_c) __attribute__((always_inline)) {
     if (T > 0 && t <= T) {
       const bool real = t < T;
-      d_cur = real ? d_next : 0u;
+      if constexpr (GS) {
+        w_cur = w_next;
+        d_cur = real ? (((w_cur >> psa_sched::REC_CODE_SHIFT) & 3u) | ((w_cur >> (psa_sched::REC_MASKED_BIT - 2)) & 4u)) : 0u;  // level | masked << 2
+      } else {
+        d_cur = real ? d_next : 0u;
+      }
       matrix_work(
           cur_c, s, pk, alpha,
           [&]() __attribute__((always_inline)) {
-            if (d_cur & 4) mask_tile(t, s);
+            if (d_cur & 4) {
+              if constexpr (GS) mask_tile_rec(t, s);
+              else mask_tile(t, s);
+            }
           },
           [&](int st) __attribute__((always_inline)) {
             if (st >= HOOK0 && st - HOOK0 < HEAD_PIECES) head_piece(st - HOOK0, s, real);
@@ -697,7 +812,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   // V_t: the vector phase.  K buffer t&1 and V buffer (t-1)&1 were last read in M_t: V(t+1) (described by ts) and
   // K(t+2) (ts2, looked up in the first half of this phase) go there, one copy instruction per 4 exponentials so
   // that the copy unit never makes the wave wait.
-  auto valu_phase = [&](int t, auto cur_c) __attribute__((always_inline)) {
+  auto valu_phase_map = [&](int t, auto cur_c) __attribute__((always_inline)) {
     constexpr int CUR = decltype(cur_c)::value;
     if (t < T) {
       const int tn = t + 2 < T ? t + 2 : T_last;
@@ -740,6 +855,49 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       ts = ts2;
       l_run = l_run * alpha + lsum;
     }
+  };
+  // The same with a prebuilt schedule: V(t+1) is described by w_v, K(t+2) by w_k; the word of tile t+3 is fetched here
+  // (one scalar load) and is complete before the phase ends.
+  auto valu_phase_rec = [&](int t, auto cur_c) __attribute__((always_inline)) {
+    constexpr int CUR = decltype(cur_c)::value;
+    if (t < T) {
+      const uint32_t w3 = *wp;
+      wp += 4;
+      bool rag = false;
+      const char* src_v = quarter_src(st_v, false, w_v, rag);
+      const char* src_k = quarter_src(st_k, true, w_k, rag);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1), V(t) of this wave have landed (visible to the group after the next barrier)
+      float lsum = 0.f;
+      if (!rag) {
+        static_for<8>([&](auto cc) __attribute__((always_inline)) {
+          constexpr int c = decltype(cc)::value;
+          float x0;
+          if constexpr (c < 4) x0 = issue_s_fma(src_v, IC<(2 + (CUR ^ 1)) * F_TILE>{}, IC<c>{}, s[c >> 2][(c & 3) * 4], nb);
+          else x0 = issue_s_fma(src_k, IC<CUR * F_TILE>{}, IC<c - 4>{}, s[c >> 2][(c & 3) * 4], nb);
+          prob4x(s[c >> 2], (c & 3) * 4, nb, pk[c >> 2] + (c & 3) * 2, lsum, x0);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      } else {
+        static_for<8>([&](auto cc) __attribute__((always_inline)) {
+          constexpr int c = decltype(cc)::value;
+          if constexpr (c < 4) issue_clamped(st_v.base, w_v, IC<(2 + (CUR ^ 1)) * F_TILE>{}, IC<c>{});
+          else issue_clamped(st_k.base, w_k, IC<CUR * F_TILE>{}, IC<c - 4>{});
+          prob4(s[c >> 2], (c & 3) * 4, nb, pk[c >> 2] + (c & 3) * 2, lsum);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
+      w_next = w_v;
+      w_v = w_k;
+      w_k = w3;
+      // the scalar load is awaited here, inside the phase: none stays in flight across the barrier into a matrix phase,
+      // whose staged waits on its LDS reads count on the same counter
+      asm volatile("" ::"s"(w_k));
+      l_run = l_run * alpha + lsum;
+    }
+  };
+  auto valu_phase = [&](int t, auto cur_c) __attribute__((always_inline)) {
+    if constexpr (GS) valu_phase_rec(t, cur_c);
+    else valu_phase_map(t, cur_c);
   };
   if (grp == 1) PP_BARRIER();
   for (int t = 0; t < C; t += 2) {
@@ -787,6 +945,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   }
 }
 
+
 template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
@@ -797,14 +956,15 @@ int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   return PSA_OK;
 }
 
-template <int D, int NW>
+template <int D, int NW, bool GS>
 int launch_fwd_pp(FwdParams& p, int Nk, hipStream_t stream) {
-  const size_t sched = (((size_t)p.max_tiles * 8 + (size_t)Nk * 2) + 15) & ~(size_t)15;
+  // with a prebuilt schedule the groups keep nothing but their tile buffers in LDS
+  const size_t sched = GS ? 0 : ((((size_t)p.max_tiles * 8 + (size_t)Nk * 2) + 15) & ~(size_t)15);
   p.grp_bytes = (int)(4 * psa_tiles::LtGeom<D>::TILE + sched);
   const size_t shmem = 2 * (size_t)p.grp_bytes;
-  if (hipFuncSetAttribute((const void*)psa_fwd_pp_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+  if (hipFuncSetAttribute((const void*)psa_fwd_pp_kernel<D, NW, GS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
     return PSA_ERR_LAUNCH;
-  hipLaunchKernelGGL((psa_fwd_pp_kernel<D, NW>), dim3((unsigned)((p.wg_chunk / 2) * p.wg_groups)), dim3(2 * NW * 64), shmem, stream, p);
+  hipLaunchKernelGGL((psa_fwd_pp_kernel<D, NW, GS>), dim3((unsigned)((p.wg_chunk / 2) * p.wg_groups)), dim3(2 * NW * 64), shmem, stream, p);
   return PSA_OK;
 }
 // LDS bytes the two-group kernel needs (tile buffers and schedule of both groups + its static tables)
@@ -825,7 +985,7 @@ extern "C" int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m) {
 static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool,
                     const void* map, int map_elem_bytes, psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L,
                     int D, int block_m, int block_n, float sm_scale, int causal, void* workspace, psa_stream_t stream,
-                    const int32_t* q_index = nullptr) {
+                    const int32_t* q_index = nullptr, const void* schedule = nullptr) {
   PSA_REQUIRE(q.ptr && k.ptr && v.ptr && out.ptr, PSA_ERR_ARG, "psa_fwd: null pointer");
   PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_fwd: pooled K/V required with a level map");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
@@ -875,6 +1035,31 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
   if (two_group) p.wg_chunk = (p.wg_chunk + 1) & ~1;  // pairs never straddle two groups of rows
   p.order = nullptr;
   p.q_index = q_index;
+  p.sched_rec = nullptr; p.sched_tiles = nullptr; p.rec_stride = 0;
+  if (schedule != nullptr) {
+    // prebuilt schedule (psa_build_schedule with the same shape arguments): issue order, tiles per row, tile records
+    psa_sched::Geometry g;
+    PSA_REQUIRE(map != nullptr && psa_schedule_geometry(B, Hq, Hkv, L, D, block_m, block_n, g), PSA_ERR_UNSUPPORTED,
+                "psa_fwd: no scheduled kernel for this shape");
+    const char* base = (const char*)schedule;
+    p.wg_chunk = g.wg_chunk; p.wg_groups = g.wg_groups;
+    p.order = (const int32_t*)(base + g.lay.order_off);
+    // the record walk assumes K / V rows D elements apart (the usual layout); other layouts walk the map in the
+    // schedule's issue order
+    int rc;
+    if (k.stride_l == D && v.stride_l == D) {
+      p.sched_rec = (const u32x4*)(base + g.lay.rec_off);
+      p.sched_tiles = (const int32_t*)(base + g.lay.tiles_off);
+      p.rec_stride = g.lay.rec_stride;
+      rc = launch_fwd_pp<128, 4, true>(p, Nk, (hipStream_t)stream);
+    } else if (two_group) {
+      rc = launch_fwd_pp<128, 4, false>(p, Nk, (hipStream_t)stream);
+    } else {
+      rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
+    }
+    PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");
+    return psa_check_launch("psa_fwd");
+  }
   if (workspace != nullptr && map != nullptr && total > 8 * 32) {
     PSA_REQUIRE((uintptr_t)workspace % 4 == 0, PSA_ERR_ARG, "psa_fwd: workspace must be 4-byte aligned");
     int32_t* order = (int32_t*)workspace;
@@ -887,7 +1072,7 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
     p.order = order;
   }
   int rc;
-  if (two_group) rc = launch_fwd_pp<128, 4>(p, Nk, (hipStream_t)stream);
+  if (two_group) rc = launch_fwd_pp<128, 4, false>(p, Nk, (hipStream_t)stream);
   else if (D == 128 && block_m == 128) rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
   else if (D == 128) rc = launch_fwd<128, 2>(p, Nk, (hipStream_t)stream);
   else if (block_m == 128) rc = launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
@@ -910,6 +1095,16 @@ extern "C" int psa_fwd_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor
   PSA_REQUIRE(q_index != nullptr, PSA_ERR_ARG, "psa_fwd_indexed: null index");
   return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal,
                   workspace, stream, q_index);
+}
+
+extern "C" int psa_fwd_scheduled(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
+                                 const void* v_pool, const void* map, int map_elem_bytes, const void* schedule, psa_tensor4 out,
+                                 float* lse, int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale,
+                                 int causal, psa_stream_t stream) {
+  PSA_REQUIRE(schedule != nullptr && map != nullptr, PSA_ERR_ARG, "psa_fwd_scheduled: null schedule or map");
+  PSA_REQUIRE((uintptr_t)schedule % 16 == 0, PSA_ERR_ARG, "psa_fwd_scheduled: schedule must be 16-byte aligned");
+  return fwd_impl(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal,
+                  nullptr, stream, q_index, schedule);
 }
 
 // ---- the variant that allocates nothing ------------------------------------------------------------------

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void psa_row_cost_kernel(const void* map, int 
   }
 }
 
-// one workgroup per share: counting sort of its items by decreasing cost (order[] holds item ids, -1 past the last item)
+// one workgroup per share: stable counting sort of its items by decreasing cost (order[] holds item ids, -1 past the last item)
 __global__ __launch_bounds__(256) void psa_chunk_sort_kernel(const int32_t* cost, int total, int chunk, int32_t* order) {
   __shared__ int hist[COST_BINS];
   const int x = blockIdx.x, tid = threadIdx.x;
@@ -91,8 +91,30 @@ __global__ __launch_bounds__(256) void psa_chunk_sort_kernel(const int32_t* cost
     }
   }
   __syncthreads();
-  for (int i = tid; i < chunk; i += 256) {
-    if (r0 + i < total) order[r0 + atomicAdd(&hist[cost[r0 + i]], 1)] = r0 + i;
+  // stable fill (items of equal cost keep their index order, so the issue order is the same in every run): 256 items at
+  // a time, an item's slot = start of its bin + the number of earlier items of the same cost
+  __shared__ int blk_cost[256];
+  for (int i0 = 0; i0 < chunk; i0 += 256) {
+    const int i = i0 + tid;
+    const bool ok = i < chunk && r0 + i < total;
+    const int c = ok ? cost[r0 + i] : -1;
+    blk_cost[tid] = c;
+    __syncthreads();
+    int before = 0, after = 0;
+    if (ok) {
+      for (int j = 0; j < 256; ++j) {
+        const bool same = blk_cost[j] == c;
+        before += (same && j < tid) ? 1 : 0;
+        after += (same && j > tid) ? 1 : 0;
+      }
+    }
+    const int pos = ok ? hist[c] + before : 0;
+    __syncthreads();
+    if (ok) {
+      order[r0 + pos] = r0 + i;
+      if (after == 0) hist[c] = pos + 1;
+    }
+    __syncthreads();
   }
   // ids past the last row of the last share
   const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;

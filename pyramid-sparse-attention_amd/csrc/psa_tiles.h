@@ -316,7 +316,7 @@ __device__ __forceinline__ const char* uniform_ptr(const char* p) {  // tells th
 __device__ __forceinline__ void lds_copy16(const char* sbase, uint32_t voff, uint32_t lds_addr) {
   sbase = uniform_ptr(sbase);
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 // the same with the target given as a uniform LDS address plus a compile-time byte offset (M0 = lds_base + OFF in one
 // scalar instruction) and the lane offset row * str + chunk computed between the write of M0 and the copy (the
@@ -330,12 +330,40 @@ __device__ __forceinline__ void lds_copy16_row(const char* sbase, uint32_t row, 
   asm volatile("s_add_u32 m0, %1, %6\n\tv_mad_u32_u24 %0, %2, %3, %4\n\tglobal_load_lds_dwordx4 %0, %5"
                : "=&v"(voff)
                : "s"(lds_base), "v"(row), "s"(str), "v"(chunk), "s"(sbase), "n"(OFF)
-               : "memory", "scc");
+               : "memory", "scc", "m0");
+}
+// the same with every address part but the lane offset in scalar registers: sbase is the (uniform) source of lane
+// offset 0 and immediate 0, voff the lane's byte offset; no vector instruction per copy.  The instruction's immediate
+// offset IMM is added to the global AND to the LDS address, so M0 gets the target minus IMM.
+template <int OFF, int IMM>
+__device__ __forceinline__ void lds_copy16_imm(const char* sbase, uint32_t voff, uint32_t lds_base) {
+  static_assert(IMM >= 0 && IMM < 4096 && OFF >= IMM, "immediate offset range");
+  sbase = uniform_ptr(sbase);
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_add_u32 m0, %1, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2 offset:%4"
+               :
+               : "v"(voff), "s"(lds_base), "s"(sbase), "n"(OFF - IMM), "n"(IMM)
+               : "memory", "scc", "m0");
+}
+// the same with a multiply-add a * b + c (a uniform) in the wait state between the write of M0 and the copy, where the
+// hardware needs an instruction anyway: the caller passes one that it has to execute in any case
+template <int OFF, int IMM>
+__device__ __forceinline__ float lds_copy16_imm_fma(const char* sbase, uint32_t voff, uint32_t lds_base, float a, float b, float c) {
+  static_assert(IMM >= 0 && IMM < 4096 && OFF >= IMM, "immediate offset range");
+  sbase = uniform_ptr(sbase);
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  a = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, a)));
+  float r;
+  asm volatile("s_add_u32 m0, %2, %4\n\tv_fma_f32 %0, %6, %7, %8\n\tglobal_load_lds_dwordx4 %1, %3 offset:%5"
+               : "=&v"(r)
+               : "v"(voff), "s"(lds_base), "s"(sbase), "n"(OFF - IMM), "n"(IMM), "s"(a), "v"(b), "v"(c)
+               : "memory", "scc", "m0");
+  return r;
 }
 // the same with a full per-lane address
 __device__ __forceinline__ void lds_copy16_addr(const char* vaddr, uint32_t lds_addr) {
   lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(vaddr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(vaddr) : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(PSA_LDS(const void))(p); }
 

@@ -87,6 +87,13 @@ SIGNATURES = {
          c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     ),
     "psa_fwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int]),
+    "psa_schedule_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "psa_build_schedule": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "psa_fwd_scheduled": (
+        c_int,
+        [Tensor4, c_void_p, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, c_void_p, Tensor4, c_void_p, c_int, c_int, c_int,
+         c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    ),
     "psa_fwd_noalloc": (
         c_int,
         [Tensor4, Tensor4, Tensor4, c_void_p, c_void_p, c_void_p, c_int, Tensor4, c_void_p, c_int, c_int, c_int, c_int,

@@ -378,6 +378,29 @@ def density(level_map_: torch.Tensor, causal: bool = False) -> torch.Tensor:
 
 
 # ----------------------------------------------------------------------------- attention forward
+def build_schedule(level_map_: torch.Tensor, Hkv: int, L: int, D: int, block_m: int, block_n: int, causal: bool = False,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Tile schedule of a level map [B, Hq, Mq, Nk] (int8 / int32): a uint8 buffer for sparse_attention_fwd(schedule=...).
+    Exists for D = 128 and 128 x 128 blocks (ValueError otherwise)."""
+    _require_gpu(level_map_)
+    if level_map_.dtype not in (torch.int8, torch.int32) or not level_map_.is_contiguous():
+        raise ValueError("level map must be a contiguous int8/int32 tensor")
+    B, Hq, Mq, Nk = level_map_.shape
+    if Mq != -(-L // block_m) or Nk != -(-L // block_n):
+        raise ValueError("level map shape does not match L and the block sizes")
+    n = lib.psa_schedule_bytes(B, Hq, Hkv, L, D, block_m, block_n)
+    if n <= 0:
+        raise ValueError("no tile schedule for D=%d, block_m=%d, block_n=%d" % (D, block_m, block_n))
+    if out is None:
+        out = torch.empty(n, dtype=torch.uint8, device=level_map_.device)
+    elif out.dtype != torch.uint8 or out.numel() < n or not out.is_contiguous() or out.device != level_map_.device:
+        raise ValueError("schedule buffer must be a contiguous uint8 tensor of at least %d bytes" % n)
+    with torch.cuda.device(level_map_.device):
+        check(lib.psa_build_schedule(_ptr(level_map_), level_map_.element_size(), _ptr(out), B, Hq, Hkv, L, D, block_m, block_n,
+                                     int(causal), _stream(level_map_)), "psa_build_schedule")
+    return out
+
+
 def sparse_attention_fwd(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -392,12 +415,15 @@ def sparse_attention_fwd(
     out: Optional[torch.Tensor] = None,
     balance: bool = True,
     q_index: Optional[torch.Tensor] = None,
+    schedule=None,
 ):
     """Pyramid sparse attention forward.  level_map_ None = dense attention.  Returns out (dtype and
     shape of q) or (out, lse fp32 [B,H,L], (k_pool, v_pool)).  balance=True issues the rows of the map
     longest first (same results, shorter tail).  q_index (int32 permutation [L]): k, v, the pools and the map are in
     the re-ordered token order, q is in the original order and read through the index (position i = row q_index[i]),
-    and out / lse come back in the original order (row q_index[i] = result of position i)."""
+    and out / lse come back in the original order (row q_index[i] = result of position i).  schedule: a tile schedule
+    built from level_map_ with build_schedule (reused across calls on the same map), None to build it here where the
+    shape has one, False to walk the map itself."""
     _require_gpu(q, k, v, level_map_, q_index)
     in_dtype = q.dtype
     qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
@@ -422,16 +448,28 @@ def sparse_attention_fwd(
     else:
         o = out
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
-    ws = None
-    if level_map_ is not None and balance:
-        ws = torch.empty(lib.psa_fwd_workspace_bytes(B, Hq, L, block_m) // 4, dtype=torch.int32, device=q.device)
-    tail = (_t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_), 1 if level_map_ is None else level_map_.element_size(), _t4(o),
-            _ptr(lse), B, Hq, Hkv, L, D, block_m, block_n, sm_scale, int(causal), _ptr(ws), _stream(q))
-    with torch.cuda.device(q.device):
-        if q_index is None:
-            check(lib.psa_fwd(_t4(qb), *tail), "psa_fwd")
-        else:
-            check(lib.psa_fwd_indexed(_t4(qb), _ptr(_check_index(q_index, L)), *tail), "psa_fwd_indexed")
+    if q_index is not None:
+        q_index = _check_index(q_index, L)
+    n_sched = lib.psa_schedule_bytes(B, Hq, Hkv, L, D, block_m, block_n) if (level_map_ is not None and balance and schedule is not False) else 0
+    if n_sched > 0:
+        # the map's tile schedule is built once (one pass over the map) and walked by the kernel
+        if not isinstance(schedule, torch.Tensor):
+            schedule = build_schedule(level_map_, Hkv, L, D, block_m, block_n, causal)
+        with torch.cuda.device(q.device):
+            check(lib.psa_fwd_scheduled(_t4(qb), _ptr(q_index), _t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_),
+                                        level_map_.element_size(), _ptr(schedule), _t4(o), _ptr(lse), B, Hq, Hkv, L, D, block_m, block_n,
+                                        sm_scale, int(causal), _stream(q)), "psa_fwd_scheduled")
+    else:
+        ws = None
+        if level_map_ is not None and balance:
+            ws = torch.empty(lib.psa_fwd_workspace_bytes(B, Hq, L, block_m) // 4, dtype=torch.int32, device=q.device)
+        tail = (_t4(kb), _t4(vb), _ptr(kp), _ptr(vp), _ptr(level_map_), 1 if level_map_ is None else level_map_.element_size(), _t4(o),
+                _ptr(lse), B, Hq, Hkv, L, D, block_m, block_n, sm_scale, int(causal), _ptr(ws), _stream(q))
+        with torch.cuda.device(q.device):
+            if q_index is None:
+                check(lib.psa_fwd(_t4(qb), *tail), "psa_fwd")
+            else:
+                check(lib.psa_fwd_indexed(_t4(qb), _ptr(q_index), *tail), "psa_fwd_indexed")
     res = o if in_dtype == torch.bfloat16 else o.to(in_dtype)
     if return_lse:
         return res, lse, (kp, vp)
