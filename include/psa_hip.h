@@ -86,6 +86,15 @@ int psa_estimate_sampled(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, con
                          int block_m, int block_n, int keep_m, int keep_n, float sm_scale,
                          int out_rows, int out_cols, psa_stream_t stream);
 
+/* Draws the estimator's sampling offsets on the device, in one launch: off_q [B*Hq, keep_m] and off_k [B*Hkv, keep_n]
+ * int32, per (batch, head) the positions of the keep largest of `block` uniform random numbers in decreasing order of
+ * the numbers (distinct offsets in 0 .. block-1; every block of a head uses the same offsets).  The numbers come from a
+ * counter-based generator keyed on `seed`: the same seed gives the same offsets, nothing is read from or written to
+ * the host.  bh_q = B * Hq, bh_kv = B * Hkv; blocks of at most 128 tokens.
+ * Replaces the rand -> topk of _random_sample_tokens: reference src/psa_triton/attention.py:128-133. */
+int psa_draw_sample_offsets(int32_t* off_q, int32_t* off_k, int bh_q, int bh_kv, int block_m, int keep_m, int block_n,
+                            int keep_n, uint64_t seed, psa_stream_t stream);
+
 /* Scores -> level map.  One row = one (b, h, q-block).  Items are (level, upper bound) in the order
  * the reference walks them: dict order for PSA_MODE_TOPK, ascending upper bound (stable) for
  * PSA_MODE_THRESHOLDBOUND - the caller passes them already in that order.  align_div = block_n/tile_n.

@@ -87,6 +87,10 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return lo + hi;
 }
 
+// Row of a token index (token re-ordering), never out of bounds: a value outside 0 .. L-1 - the caller's mistake, the
+// Python mirror rejects such an index - reads row 0 / L-1 instead of faulting.
+__device__ __forceinline__ int clamp_row(int v, int L) { return v < 0 ? 0 : (v < L ? v : L - 1); }
+
 // level value (0,1,2,4,8) of a map element of 1 or 4 bytes
 __device__ __forceinline__ int load_map(const void* map, int64_t idx, int elem_bytes) {
   return elem_bytes == 1 ? (int)((const int8_t*)map)[idx] : ((const int32_t*)map)[idx];

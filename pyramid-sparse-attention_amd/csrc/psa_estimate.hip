@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
       int src = sampled_src(row0 + rs * 32 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
-      if (p.q_index != nullptr) src = p.q_index[src];
+      if (p.q_index != nullptr) src = clamp_row(p.q_index[src], p.Lq);
       const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) qf[rs][kk] = *(const bf16x8*)(qp + kk * 16);

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   bf16x8 qf[KK];
   {
     int qr = q_idx < P_L ? q_idx : P_L - 1;
-    if (p.q_index != nullptr) qr = p.q_index[qr];
+    if (p.q_index != nullptr) qr = clamp_row(p.q_index[qr], P_L);
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
@@ -339,7 +339,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   const float inv = 1.0f / l_safe;
   if (p.lse != nullptr && hh == 0 && q_idx < P_L) {
     // natural-log domain: m*ln2 + ln(max(l, 1e-8))
-    p.lse[((int64_t)b * p.Hq + h) * P_L + (p.q_index != nullptr ? p.q_index[q_idx] : q_idx)] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+    const int lrow = p.q_index != nullptr ? p.q_index[q_idx] : q_idx;  // (a row outside 0 .. L-1 is not stored)
+    if ((unsigned)lrow < (unsigned)P_L) p.lse[((int64_t)b * p.Hq + h) * P_L + lrow] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
   }
   __syncthreads();  // everyone is done with the last K/V tile
   unsigned char* Os = smem;
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
     const int row = I * BM + r;
     if (row < P_L) {
       const int orow = p.q_index != nullptr ? p.q_index[row] : row;
-      *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+      if ((unsigned)orow < (unsigned)P_L) *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
     }
   }
 }
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   bf16x8 qf[KK];
   {
     int qr = q_idx < P_L ? q_idx : P_L - 1;
-    if (p.q_index != nullptr) qr = p.q_index[qr];
+    if (p.q_index != nullptr) qr = clamp_row(p.q_index[qr], P_L);
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
@@ -917,7 +918,8 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   const float l_safe = fmaxf(l_tot, 1e-8f);
   const float inv = 1.0f / l_safe;
   if (active && p.lse != nullptr && hh == 0 && q_idx < P_L) {
-    p.lse[((int64_t)b * p.Hq + h) * P_L + (p.q_index != nullptr ? p.q_index[q_idx] : q_idx)] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
+    const int lrow = p.q_index != nullptr ? p.q_index[q_idx] : q_idx;  // (a row outside 0 .. L-1 is not stored)
+    if ((unsigned)lrow < (unsigned)P_L) p.lse[((int64_t)b * p.Hq + h) * P_L + lrow] = (m_run + fast_log2(l_safe)) * 0.6931471805599453f;
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // the last (repeated) tile copies land in the buffers that now stage O
   __syncthreads();
@@ -939,7 +941,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       const int row = I * BM + r;
       if (row < P_L) {
         const int orow = p.q_index != nullptr ? p.q_index[row] : row;
-        *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
+        if ((unsigned)orow < (unsigned)P_L) *(u32x4*)(ob + (int64_t)orow * p.o_sl + ch * 8) = *(const u32x4*)(Os + r * OST + ch * 16);
       }
     }
   }

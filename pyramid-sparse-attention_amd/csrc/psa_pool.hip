@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void psa_pool_kernel(PoolParams p) {
     int64_t row = g * 8 + i;
     const bool real = row < p.L;
     row = real ? row : (int64_t)(p.L - 1);
-    const int64_t srow = INDEXED ? (int64_t)p.index[row] : row;
+    const int64_t srow = INDEXED ? (int64_t)clamp_row(p.index[row], p.L) : row;
     u32x4 w = *(const u32x4*)(src + srow * sl);
     if (INDEXED && real)
       __builtin_nontemporal_store(w, (u32x4*)(p.ord[which] + b * p.ob[which] + h * p.oh[which] + row * p.ol[which] + c * 8));

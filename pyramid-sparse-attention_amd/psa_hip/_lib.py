@@ -5,7 +5,7 @@ ImportError with the command that builds it.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpsa_hip.so")
@@ -42,6 +42,7 @@ SIGNATURES = {
          c_int, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int, c_int, c_double,
          c_void_p],
     ),
+    "psa_draw_sample_offsets": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_uint64, c_void_p]),
     "psa_level_map": (
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, POINTER(c_int32), POINTER(c_double), c_int,

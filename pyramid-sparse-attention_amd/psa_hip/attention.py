@@ -69,14 +69,18 @@ class PSAConfig:
 
 def draw_sample_offsets(B: int, H: int, block: int, keep: int, device, generator=None) -> torch.Tensor:
     """`keep` distinct in-block offsets per (b, h), int32 [B,H,keep]; every block of a head uses the
-    same offsets.  reference: src/psa_triton/attention.py:132-133 (rand -> topk)."""
-    if generator is not None and generator.device.type != "cpu":
-        r = torch.rand(B, H, 1, block, device=device, generator=generator)
-        return torch.topk(r, keep, dim=3).indices.view(B, H, keep).to(torch.int32).contiguous()
-    # Drawn on the host (default or given CPU generator): B*H*block numbers.  On the device the rand -> topk ->
-    # convert chain costs five launches and ~55 us per call, twice per layer, next to a 1 ms layer.
-    r = torch.rand(B, H, block, generator=generator)
-    return torch.topk(r, keep, dim=2).indices.to(torch.int32).contiguous().to(device, non_blocking=True)
+    same offsets.  reference: src/psa_triton/attention.py:132-133 (rand -> topk).  With a torch generator the draw is
+    torch's own rand -> topk on that generator's device; without one it is a single kernel on the GPU
+    (ops.draw_sample_offsets: both tensors of a layer in one launch, nothing crosses the host)."""
+    if generator is not None:
+        r = torch.rand(B, H, block, device=generator.device, generator=generator)
+        return torch.topk(r, keep, dim=2).indices.to(torch.int32).contiguous().to(device)
+    return ops.draw_sample_offsets(B, H, H, block, keep, block, keep, device)[0]
+
+
+def draw_layer_offsets(B: int, Hq: int, Hkv: int, block_m: int, block_n: int, device):
+    """(off_q, off_k) of one layer: a quarter of each block, drawn on the device in one launch."""
+    return ops.draw_sample_offsets(B, Hq, Hkv, block_m, block_m // 4, block_n, block_n // 4, device)
 
 
 def _compute_attention_pooling(q, k, v, config, sample_offsets=None):
@@ -89,8 +93,7 @@ def _compute_attention_pooling(q, k, v, config, sample_offsets=None):
     if config.use_sim_mask:
         sim_cap = calc_k_similarity(k, config.block_n, config)
     if sample_offsets is None:
-        off_q = draw_sample_offsets(B, H, config.block_m, keep_m, q.device)
-        off_k = draw_sample_offsets(B, Hkv, config.block_n, keep_n, k.device)
+        off_q, off_k = draw_layer_offsets(B, H, Hkv, config.block_m, config.block_n, q.device)
     else:
         off_q, off_k = sample_offsets
     pooling = ops.estimate_sampled(q, k, off_q, off_k, config.block_m, config.block_n, keep_m, keep_n, q.size(-1) ** -0.5)
@@ -127,8 +130,7 @@ class PSAAttention(nn.Module):
             # inference: the stages back to back with a dense int8 level map (same levels as the mask formats)
             if self.sample_offsets is None:
                 B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
-                off_q = draw_sample_offsets(B, H, config.block_m, config.block_m // 4, q.device)
-                off_k = draw_sample_offsets(B, Hkv, config.block_n, config.block_n // 4, k.device)
+                off_q, off_k = draw_layer_offsets(B, H, Hkv, config.block_m, config.block_n, q.device)
             else:
                 off_q, off_k = self.sample_offsets
             cap = calc_k_similarity(k, config.block_n, config) if config.use_sim_mask else None

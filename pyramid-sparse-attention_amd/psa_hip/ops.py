@@ -63,10 +63,39 @@ def pool_kv(k: torch.Tensor, v: torch.Tensor, block_n: int, out: Optional[Tuple[
     return kp, vp
 
 
-def _check_index(index: torch.Tensor, L: int) -> torch.Tensor:
+_VALID_INDEX: Dict[Tuple[int, int, int, int], bool] = {}
+
+
+def validate_token_index(index: torch.Tensor, L: int) -> None:
+    """Raises ValueError unless index is a permutation of 0 .. L-1 (works on CPU and GPU tensors; one small reduction)."""
     if index.dtype != torch.int32 or index.dim() != 1 or index.numel() != L:
         raise ValueError("index must be a 1-D int32 tensor with one entry per token (%d)" % L)
-    return index.contiguous()
+    if L == 0:
+        return
+    idx = index.to(torch.int64)
+    if int(idx.min()) < 0 or int(idx.max()) >= L:
+        raise ValueError("token index has entries outside 0 .. %d" % (L - 1))
+    seen = torch.zeros(L, dtype=torch.int32, device=index.device)
+    seen.index_fill_(0, idx, 1)
+    if int(seen.sum()) != L:
+        raise ValueError("token index is not a permutation of 0 .. %d: %d positions are never written" % (L - 1, L - int(seen.sum())))
+
+
+def _check_index(index: torch.Tensor, L: int) -> torch.Tensor:
+    """A token index the kernels can use: int32, one entry per token, a permutation of 0 .. L-1.  A bad entry would make
+    a kernel read or write another row (the kernels clamp reads and drop stores outside the tensor, so nothing faults,
+    but rows of the output would stay unwritten): the contents are checked once per index tensor (keyed on its storage
+    and version, so an index built once per model costs one check)."""
+    if index.dtype != torch.int32 or index.dim() != 1 or index.numel() != L:
+        raise ValueError("index must be a 1-D int32 tensor with one entry per token (%d)" % L)
+    index = index.contiguous()
+    key = (index.data_ptr(), index._version, L, index.device.index if index.device.index is not None else -1)
+    if key not in _VALID_INDEX:
+        validate_token_index(index, L)
+        if len(_VALID_INDEX) > 64:
+            _VALID_INDEX.clear()
+        _VALID_INDEX[key] = True
+    return index
 
 
 def pool_kv_indexed(k: torch.Tensor, v: torch.Tensor, index: torch.Tensor, block_n: int):
@@ -100,6 +129,28 @@ def pool_levels(pool: torch.Tensor, B: int, H: int, L: int, D: int, block_n: int
 
 
 # ----------------------------------------------------------------------------- estimator
+_DRAWS = [0]
+
+
+def draw_sample_offsets(B: int, Hq: int, Hkv: int, block_m: int, keep_m: int, block_n: int, keep_n: int, device,
+                        seed: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(off_q [B,Hq,keep_m], off_k [B,Hkv,keep_n]) int32, drawn on the device in one launch (no host round trip): per
+    (b, h) `keep` distinct in-block offsets, the same for every block of the head.  seed None: a new draw per call,
+    derived from torch's seed (torch.manual_seed makes a run reproducible) and a call counter."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("psa_hip operators run on the GPU only; there is no CPU path")
+    if seed is None:
+        _DRAWS[0] += 1
+        seed = (torch.initial_seed() * 0x9E3779B97F4A7C15 + _DRAWS[0]) & 0xFFFFFFFFFFFFFFFF
+    off_q = torch.empty(B, Hq, keep_m, dtype=torch.int32, device=device)
+    off_k = torch.empty(B, Hkv, keep_n, dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        check(lib.psa_draw_sample_offsets(_ptr(off_q), _ptr(off_k), B * Hq, B * Hkv, block_m, keep_m, block_n, keep_n,
+                                          int(seed) & 0xFFFFFFFFFFFFFFFF, _stream(off_q)), "psa_draw_sample_offsets")
+    return off_q, off_k
+
+
 def estimate_sampled(
     q: torch.Tensor,
     k: torch.Tensor,

@@ -15,7 +15,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .attention import draw_sample_offsets
+from .attention import draw_layer_offsets, draw_sample_offsets
 from .kernels.calc_ksim_kernel import calc_k_similarity
 from .kernels.psa_kernel import sparse_attention_factory as psa_sparse_attention
 from .kernels.psa_kernel_legacy import sparse_attention_factory as psa_sparse_attention_legacy
@@ -70,8 +70,7 @@ def efficient_attn_with_pooling(q, k, v, config, num_keep_m=32, num_keep_n=32, s
     sim_cap = calc_k_similarity(k, config.block_n, config) if getattr(config, "use_sim_mask", True) else None
     B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
     if sample_offsets is None:
-        off_q = draw_sample_offsets(B, H, config.block_m, num_keep_m, q.device)
-        off_k = draw_sample_offsets(B, Hkv, config.block_n, num_keep_n, k.device)
+        off_q, off_k = ops.draw_sample_offsets(B, H, Hkv, config.block_m, num_keep_m, config.block_n, num_keep_n, q.device)
     else:
         off_q, off_k = sample_offsets
     pooling = ops.estimate_sampled(q, k, off_q, off_k, config.block_m, config.block_n, num_keep_m, num_keep_n, q.size(-1) ** -0.5,
@@ -207,8 +206,7 @@ class PyramidSparseAttention(nn.Module):
         cfg = self.config
         B, H, Hkv = q.shape[0], q.shape[1], k.shape[1]
         if self.sample_offsets is None:
-            off_q = draw_sample_offsets(B, H, cfg.block_m, cfg.block_m // 4, q.device)
-            off_k = draw_sample_offsets(B, Hkv, cfg.block_n, cfg.block_n // 4, k.device)
+            off_q, off_k = draw_layer_offsets(B, H, Hkv, cfg.block_m, cfg.block_n, q.device)
         else:
             off_q, off_k = self.sample_offsets
         if cfg.mask_mode not in ("topk", "thresholdbound"):

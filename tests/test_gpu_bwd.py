@@ -73,6 +73,26 @@ def test_bwd_each_level_alone_and_unused_blocks():
     assert torch.all(dk[0, 0, :256] == 0) and torch.all(dv[0, 0, :256] == 0)  # kv-blocks nobody retains
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_bwd_more_than_256_rows_ordered_walks(causal):
+    """272 rows of the map (B 2, 4 query heads on 2 kv heads, 34 q-blocks of 128, ragged last block): the dQ walk runs in
+    its longest-first issue order (chunk sort, -1 padding, early return of the padded entries), the level-0 dK/dV walk
+    writes bf16 directly.  Random map with skipped blocks and rows that retain nothing, against the oracle."""
+    B, Hq, Hkv, L = 2, 4, 2, 128 * 33 + 40
+    Mq = 34
+    lmap = random_map(B, Hq, Mq, Mq, 91, p=(0.55, 0.15, 0.1, 0.1, 0.1), ensure_row=False)
+    if causal:
+        lmap[..., np.arange(Mq), np.arange(Mq)] = 1
+    else:
+        lmap[0, 1, 5] = 0   # rows without keys
+        lmap[1, 3, 33] = 0  # ... incl. the ragged last q-block
+        lmap[1, 0, :, 7] = 0  # a kv-block nobody retains
+    assert B * Hq * Mq > 256
+    dq, dk, dv, _ = run_bwd(B, Hq, Hkv, L, 128, 128, 128, causal, seed=92, lmap=lmap)
+    if not causal:
+        assert torch.all(dq[0, 1, 5 * 128:6 * 128] == 0) and torch.all(dq[1, 3, 33 * 128:] == 0)
+
+
 def test_bwd_all_ones_matches_sdpa_autograd():
     from psa_hip import ops
 

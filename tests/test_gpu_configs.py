@@ -127,6 +127,36 @@ def test_c2_wan_layer_reduced_vs_oracle():
     assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
 
 
+def test_c2_wan_layer_full_size_vs_oracle():
+    """The headline workload at its own size: B 1, H 12, N 32760 (21x30x52 grid), D 128, blocks of 128, thresholdbound
+    calibrated to ~90 % sparsity, rows issued longest first through the tile schedule - the whole layer operator.
+    Scores of all 12 heads against the oracle (rtol 2e-4), the level map of all heads bit for bit from the GPU's
+    scores, and the output of two heads - every q-block, so every phase of the row dealing and both ends of the
+    longest-first order - against the oracle's block walk on the host (max-abs 2e-2, mean-abs 2e-3)."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    B, H, D, bm, bn, tn = 1, 12, 128, 128, 128, 32
+    q, k, v = make_qkv(B, H, H, (21, 30, 52), D, seed=1234)
+    L = q.shape[2]
+    assert L == 32760
+    oq, ok = sample_offsets(B, H, bm, 32, 1244), sample_offsets(B, H, bn, 32, 1245)
+    qd, kd, vd, oqd, okd = (t.to(dev()) for t in (q, k, v, oq, ok))
+    scores = ops.estimate_sampled(qd, kd, oqd, okd, bm, bn, 32, 32)
+    ratios = calibrate(ops, scores, 0.90, bn, tn)
+    out, mp = ops.psa_layer_fwd(qd, kd, vd, oqd, okd, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+    torch.cuda.synchronize()
+    assert abs(float(ops.density(mp)[-1]) - 0.10) < 0.01
+    torch.set_num_threads(min(torch.get_num_threads(), 16))
+    heads = [1, 10]  # (one head per half of the phases of the row dealing)
+    np.testing.assert_allclose(scores.cpu().numpy(), O.estimate_sampled(q, k, bm, bn, oq, ok).numpy(), rtol=2e-4, atol=1e-9)
+    ref_map = O.level_map(scores.cpu().numpy(), ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn)
+    assert np.array_equal(mp.cpu().numpy(), ref_map)
+    ref, _ = O.psa_attention_blockwalk(q[:, heads], k[:, heads], v[:, heads], ref_map[:, heads], bm, bn)
+    mx, mean = attn_errors(out[:, heads], ref)
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+
+
 # ------------------------------------------------------------------------------------------------ c3
 def test_c3_cogvideox_reduced_end_to_end_vs_oracle():
     """B 2 (CFG), D 64, blocks of 128, 226 text tokens after a 5x12x20 video grid, top-k with the ratios of the
@@ -267,3 +297,30 @@ def test_c5_reduced_prefill_vs_oracle():
     ref, _ = O.psa_attention_blockwalk(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), ref_map, 128, 128, causal=True)
     mx, mean = attn_errors(out, ref)
     assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+
+
+def test_c5_gqa_ratio_7_forward_lse_backward_vs_oracle():
+    """The head ratio of the causal prefill configuration (28 query heads on 4 kv heads = 7 per kv head) at 14 / 2 heads
+    and 2048 tokens: causal forward, lse and backward on a random map with skips against the oracle (the backward's
+    dK / dV sum seven query heads per kv head)."""
+    from psa_hip import ops
+    from gpu_util import random_map, rnd
+
+    B, Hq, Hkv, L, D = 1, 14, 2, 2048, 128
+    q, k, v = rnd(B, Hq, L, D, seed=71), rnd(B, Hkv, L, D, seed=72), rnd(B, Hkv, L, D, seed=73)
+    do = rnd(B, Hq, L, D, seed=74, scale=0.02)
+    lmap = random_map(B, Hq, 16, 16, 75)
+    idx = np.arange(16)
+    lmap[..., idx, idx] = 1  # (the diagonal is always kept at level 1 by the causal map rules)
+    qd, kd, vd, dod, md = (t.to(dev()) for t in (q, k, v, do, torch.from_numpy(lmap)))
+    out, lse, pools = ops.sparse_attention_fwd(qd, kd, vd, md, 128, 128, causal=True, return_lse=True)
+    dq, dk, dv = ops.sparse_attention_bwd(qd, kd, vd, md, out, dod, lse, 128, 128, causal=True, pools=pools)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.psa_attention_dense(q, k, v, lmap, 128, 128, causal=True)
+    mx, mean = attn_errors(out, ref)
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+    fin = torch.isfinite(ref_lse)
+    assert float((lse.cpu().double()[fin] - ref_lse[fin]).abs().max()) <= 2e-2
+    rdq, rdk, rdv = O.psa_backward_dense(q, k, v, lmap, do, 128, 128, causal=True)
+    errs = [rel_l2(a.float().cpu(), b) for a, b in ((dq, rdq), (dk, rdk), (dv, rdv))]
+    assert max(errs) <= REL_L2, errs

@@ -103,3 +103,33 @@ def test_fused_estimate_and_map_very_wide_rows_fall_back_to_two_kernels():
     ref = ops.level_map(scores, ratios, 0, "thresholdbound", blocksize=bn, compute_tile=32, map_dtype=torch.int8)
     got = ops.estimate_sampled_map(q, k, None, None, bm, bn, 32, 8, ratios, 0, "thresholdbound", compute_tile=32, map_dtype=torch.int8)
     assert got.shape == (1, 1, 1500, 6000) and torch.equal(got, ref)
+
+
+def test_sampling_offsets_drawn_on_the_device():
+    """psa_draw_sample_offsets: per (b, h) `keep` distinct offsets inside the block, reproducible from the seed, different
+    between heads and seeds, every offset about equally likely (the reference draws rand -> topk: a uniform subset)."""
+    from psa_hip import ops
+
+    B, Hq, Hkv = 2, 48, 12
+    oq, ok = ops.draw_sample_offsets(B, Hq, Hkv, 128, 32, 64, 16, dev(), seed=1234)
+    assert oq.shape == (B, Hq, 32) and ok.shape == (B, Hkv, 16) and oq.dtype == torch.int32
+    for o, block, keep in ((oq, 128, 32), (ok, 64, 16)):
+        o = o.cpu().numpy().reshape(-1, keep)
+        assert o.min() >= 0 and o.max() < block
+        assert all(len(set(r)) == keep for r in o)          # distinct
+        assert len({tuple(r) for r in o}) == o.shape[0]      # heads differ
+    oq2, ok2 = ops.draw_sample_offsets(B, Hq, Hkv, 128, 32, 64, 16, dev(), seed=1234)
+    assert torch.equal(oq, oq2) and torch.equal(ok, ok2)
+    oq3, _ = ops.draw_sample_offsets(B, Hq, Hkv, 128, 32, 64, 16, dev(), seed=1235)
+    assert not torch.equal(oq, oq3)
+    # uniformity: 4096 heads x 32 of 128 -> every offset expected 1024 times (sd ~ 28)
+    big, _ = ops.draw_sample_offsets(64, 64, 1, 128, 32, 64, 16, dev(), seed=7)
+    cnt = np.bincount(big.cpu().numpy().reshape(-1), minlength=128)
+    assert cnt.sum() == 4096 * 32 and abs(cnt - 1024).max() < 6 * 28
+    # the first offset of a head (the largest random number) is uniform too
+    first = np.bincount(big.cpu().numpy().reshape(-1, 32)[:, 0], minlength=128)
+    assert abs(first - 32).max() < 6 * 6
+    # unseeded draws differ from call to call
+    a, _ = ops.draw_sample_offsets(1, 4, 4, 128, 32, 128, 32, dev())
+    b, _ = ops.draw_sample_offsets(1, 4, 4, 128, 32, 128, 32, dev())
+    assert not torch.equal(a, b)

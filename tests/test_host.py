@@ -198,3 +198,25 @@ def test_psa_logger_schema_and_summary(tmp_path):
         assert needle in summary, needle
     cfgj = json.load(open(tmp_path / "s" / "config.json"))
     assert cfgj["model_type"] == "wan" and cfgj["layer_num"] == 2 and cfgj["config"]["attn_impl"] == "old_mask_type"
+
+
+def test_token_index_validator_rejects_what_is_not_a_permutation():
+    """A token index that is not a permutation of 0 .. L-1 is refused on the host (the kernels clamp what they read and
+    drop what they cannot store, but rows of the output would stay unwritten)."""
+    import pytest
+    import torch
+
+    from psa_hip import ops
+
+    L = 37
+    good = torch.randperm(L, generator=torch.Generator().manual_seed(0)).to(torch.int32)
+    ops.validate_token_index(good, L)
+    for bad in (good.clone().index_fill_(0, torch.tensor([3]), L),      # past the end
+                good.clone().index_fill_(0, torch.tensor([5]), -1),     # negative
+                good.clone().index_fill_(0, torch.tensor([7]), int(good[8]))):  # repeated: one row never written
+        with pytest.raises(ValueError):
+            ops.validate_token_index(bad, L)
+    with pytest.raises(ValueError):
+        ops.validate_token_index(good.to(torch.int64), L)
+    with pytest.raises(ValueError):
+        ops.validate_token_index(good[:-1], L)

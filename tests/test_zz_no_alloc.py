@@ -1,6 +1,7 @@
-"""The allocation-free forward entry point (psa_fwd_noalloc) against psa_fwd with a workspace, through the C ABI:
-two calls in a row, the second on a smaller input, each bit-identical to the existing entry point (same kernels, the
-row-ordering scratch in the library's own device array instead of a caller workspace)."""
+"""The allocation-free forward entry point (psa_fwd_noalloc) against the forward operator, through the C ABI: two calls
+in a row, the second on a smaller input, each bit-identical to the existing entry point (the row-ordering scratch in
+the library's own device array instead of a caller workspace); the driver's free-memory figure does not move across a
+call; and the call can be captured into a HIP graph and replayed."""
 import ctypes
 
 import numpy as np
@@ -35,21 +36,56 @@ def _call_pair(B, Hq, Hkv, L, D, bm, bn, causal, seed):
     lse = torch.full((B, Hq, L), float("nan"), dtype=torch.float32, device=dev())
     t4 = lambda x: Tensor4(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2))
     p = lambda x: ctypes.c_void_p(x.data_ptr())
+
+    def call():
+        return lib.psa_fwd_noalloc(t4(q), t4(k), t4(v), p(kp), p(vp), p(m), 1, t4(out), p(lse), B, Hq, Hkv, L, D, bm, bn,
+                                   float(D ** -0.5), int(causal), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    # one warm call (the library looks its scratch array's address up once per device), then the measured one: the
+    # driver's own count of free device memory - which any hipMalloc would lower, inside the library as well as
+    # in torch - is the same before and after
+    check(call(), "psa_fwd_noalloc")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    rc = lib.psa_fwd_noalloc(t4(q), t4(k), t4(v), p(kp), p(vp), p(m), 1, t4(out), p(lse), B, Hq, Hkv, L, D, bm, bn,
-                             float(D ** -0.5), int(causal), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    check(rc, "psa_fwd_noalloc")
+    out.fill_(float("nan"))
+    lse.fill_(float("nan"))
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    free_before = torch.cuda.mem_get_info()[0]
+    check(call(), "psa_fwd_noalloc")
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert not torch.isnan(out).any() and not torch.isnan(lse).any()
     assert torch.equal(out, ref) and torch.equal(lse, ref_lse)
+    return call, out, lse, ref, ref_lse
 
 
 def test_noalloc_forward_two_calls_second_smaller():
     _call_pair(1, 5, 5, 128 * 67 + 40, 128, 128, 128, False, 3)   # 340 rows of the map
     _call_pair(1, 4, 2, 128 * 66, 128, 128, 128, True, 4)          # 264 rows: smaller, causal, grouped heads
     _call_pair(2, 3, 3, 128 * 50 + 7, 64, 128, 128, False, 5)      # the one-row kernel (head dim 64), 306 rows
+
+
+def test_noalloc_forward_under_graph_capture():
+    """What the entry point is for: captured into a HIP graph (only kernel nodes: nothing is allocated or cleared inside
+    the call) and replayed several times with eager work in between; every replay gives the eager bits."""
+    call, out, lse, ref, ref_lse = _call_pair(1, 5, 5, 128 * 67 + 40, 128, 128, 128, False, 7)
+    from psa_hip._lib import check
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            check(call(), "psa_fwd_noalloc (captured)")
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        out.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        junk = torch.randn(1 << 20, device=dev()).sum()  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref) and torch.equal(lse, ref_lse), rep
+        assert torch.isfinite(junk)
 
 
 def test_noalloc_forward_rejects_oversized_shapes():
