@@ -322,6 +322,15 @@ def main():
     per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     ms_step_median = per_step[len(per_step) // 2]
 
+    # the same layer captured into one HIP graph (kernel nodes only) and replayed
+    def layer_graph():
+        return ops.psa_layer_fwd_graph(q, k, v, off_q, off_k, ratios, mode, bm, bn, tn, return_map=True, text_length=text)
+
+    o_g, mp_g = layer_graph()
+    torch.cuda.synchronize()
+    graph_equal = bool(torch.equal(o_g, state["o"])) and bool(torch.equal(mp_g, state["mp"]))
+    t_graph, _ = time_gpu(layer_graph, max(10, min(args.steps, 100)))
+
     mp = state["mp"]
     kp, vp = ops.pool_kv(k, v, bn)
     state["s"] = ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn)
@@ -485,7 +494,8 @@ def main():
         "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
                    "sparsity": round(1 - density, 4), "mask_mode": mode, "tau": None if tau != tau else round(tau, 4)},
         "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
-                      "schedule": None if t_sched is None else round(t_sched, 4), "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4)},
+                      "schedule": None if t_sched is None else round(t_sched, 4), "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4),
+                      "layer_graph": round(t_graph, 4), "layer_graph_bit_identical": graph_equal},
         "reorder_ms": reorder,
         "preset_ms": preset,
         "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),

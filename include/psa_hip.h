@@ -40,14 +40,22 @@ extern "C" {
 
 typedef void* psa_stream_t; /* hipStream_t */
 
-/* [B, H, L, D] bf16 view; strides in elements; the D stride is 1.  Every entry point computes on bf16 operands with
- * fp32 accumulation and takes bf16 tensors only: a caller that holds fp16 / fp32 tensors (the reference accepts them)
- * rounds them to bf16 first, as the Python mirror does, and the results then carry that input rounding. */
+/* Element types.  The kernels compute in the type of their tensors, as the reference's do (tl.dot on q / k as loaded,
+ * p.to(v.dtype): reference src/psa_triton/kernels/psa_kernel.py:49-77): bf16 and fp16 operands on the matrix cores with
+ * fp32 accumulation, fp32 tensors in fp32 throughout.  All tensors of one call (and its pooled buffers) share one
+ * type.  Entry points say which types they take; the others return PSA_ERR_UNSUPPORTED. */
+#define PSA_DTYPE_BF16 0
+#define PSA_DTYPE_F16 1
+#define PSA_DTYPE_F32 2
+
+/* [B, H, L, D] view; strides in elements; the D stride is 1.  dtype: PSA_DTYPE_* (0 = bf16). */
 typedef struct psa_tensor4 {
   void* ptr;
   int64_t stride_b;
   int64_t stride_h;
   int64_t stride_l;
+  int32_t dtype;
+  int32_t reserved;
 } psa_tensor4;
 
 int psa_version(void);
@@ -156,6 +164,14 @@ int psa_estimate_xattn(psa_tensor4 q, psa_tensor4 k, float* est, void* workspace
  * after 8.  reference src/psa_triton/kernels/psa_kernel.py:207-217. */
 int psa_map_from_list(const int32_t* list, void* map_out, int map_elem_bytes, int64_t rows,
                       int width, int Nk, psa_stream_t stream);
+
+/* Dense level map [rows, Nk] -> index list [rows, Nk + 5] int32: the kv-blocks at levels 1, 2, 4, 8 and then the skipped
+ * ones, each segment followed by -1 (blocks of a level in ascending order).  A segment's length is rounded down to a
+ * multiple of ceil(level / align_div), align_div = blocksize / compute_tile, and the blocks that do not fit lead the next
+ * segment (they are pooled one level coarser), as in the reference.
+ * Replaces transfer_mask_to_new_type: reference src/psa_triton/utils/transfer_attn_to_mask.py:624-750. */
+int psa_list_from_map(const void* map, int map_elem_bytes, int32_t* list_out, int64_t rows, int Nk, int align_div,
+                      psa_stream_t stream);
 
 /* Key-similarity cap: cap_out [B, H, Nk] int32 in {1, 2, 4, 8}.  For a kv-block, sim_l = mean cosine
  * similarity of the token pairs (g*l, g*l + l-1); the cap is the largest l in {2, 4, 8} with

@@ -364,6 +364,37 @@ def list_to_dense(list_mask: np.ndarray, Nk: int) -> np.ndarray:
     return out.reshape(lead + (Nk,))
 
 
+def dense_to_list(level_map_dense: np.ndarray, blocksize: int = 32, compute_tile: int = 32) -> np.ndarray:
+    """Dense level map [..., Nk] -> index list [..., Nk + 5]: blocks at levels 1, 2, 4, 8, then the skipped ones, a -1
+    behind each segment; a segment's length is rounded down to a multiple of ceil(level / (blocksize // compute_tile))
+    and the blocks that do not fit lead the next segment.
+    reference: src/psa_triton/utils/transfer_attn_to_mask.py:624-750 (transfer_mask_to_new_type).  Blocks of a level
+    are listed in ascending order (the reference leaves the order inside a level to torch.sort)."""
+    m = np.asarray(level_map_dense)
+    lead, Nk = m.shape[:-1], m.shape[-1]
+    flat = m.reshape(-1, Nk)
+    div = max(1, blocksize // compute_tile)
+    out = np.zeros((flat.shape[0], Nk + 5), dtype=np.int32)
+    for r in range(flat.shape[0]):
+        order = [j for val in (1, 2, 4, 8) for j in range(Nk) if flat[r, j] == val]
+        order += [j for j in range(Nk) if flat[r, j] not in (1, 2, 4, 8)]
+        counts = [int((flat[r] == val).sum()) for val in (1, 2, 4, 8)]
+        counts.append(Nk - sum(counts))
+        for t, val in enumerate((1, 2, 4, 8)):
+            mult = max(1, -(-val // div))
+            rem = counts[t] % mult if mult > 1 else 0
+            counts[t] -= rem
+            counts[t + 1] += rem
+        pos, src = 0, 0
+        for t in range(5):
+            out[r, pos : pos + counts[t]] = order[src : src + counts[t]]
+            pos += counts[t]
+            src += counts[t]
+            out[r, pos] = -1
+            pos += 1
+    return out.reshape(lead + (Nk + 5,))
+
+
 def density(level_map_dense: np.ndarray) -> float:
     """mean(1/level) with skipped blocks counting 0.
     reference: src/psa_triton/utils/transfer_attn_to_mask.py:510-544."""

@@ -16,6 +16,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 #define PSA_WAVE 64
 
@@ -55,6 +59,59 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---- the 16-bit element types the MFMA kernels compute in (operands in the caller's type, fp32 accumulation) ------
+// bf16: v_mfma_f32_32x32x16_bf16; fp16: v_mfma_f32_32x32x16_f16 - same rate, same operand and accumulator layouts, so
+// a kernel is written once over one of these traits.
+#define PSA_LDS_PTR(T) __attribute__((address_space(3))) T*
+struct EtBf16 {
+  static constexpr int id = PSA_DTYPE_BF16;
+  using t = bf16_t;
+  using x8 = bf16x8;
+  static __device__ __forceinline__ float from_bits(uint32_t b16) { return bf16_bits_to_f32(b16); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+  static __device__ __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  // transposing LDS read: 4 keys of one channel
+  static __device__ __forceinline__ u32x2 read_tr(PSA_LDS_PTR(unsigned char) a) {
+    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS_PTR(bf16x4))a));
+  }
+  // acc + lo + hi of a packed pair (the rounded values)
+  static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+    const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
+  }
+};
+struct EtF16 {
+  static constexpr int id = PSA_DTYPE_F16;
+  using t = f16_t;
+  using x8 = f16x8;
+  static __device__ __forceinline__ float from_bits(uint32_t b16) { return (float)__builtin_bit_cast(f16_t, (uint16_t)b16); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));  // round to nearest even
+  }
+  static __device__ __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ u32x2 read_tr(PSA_LDS_PTR(unsigned char) a) {
+    return EtBf16::read_tr(a);  // (the transposing read moves 16-bit words whatever they hold)
+  }
+  static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+    const f16x2 ones = {(f16_t)1.0f, (f16_t)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
+  }
+};
+// calls f(trait) for a 16-bit dtype id; false for any other id
+template <class F>
+static inline bool psa_dispatch16(int dtype, F&& f) {
+  if (dtype == PSA_DTYPE_BF16) {
+    f(EtBf16{});
+    return true;
+  }
+  if (dtype == PSA_DTYPE_F16) {
+    f(EtF16{});
+    return true;
+  }
+  return false;
+}
 
 // max of three: compiles to one v_max3_f32 in translation units built without NaN semantics (the compiler then
 // needs no canonicalising pass over its inputs).  Plain C on purpose: hand-written assembly would not get the

@@ -4,7 +4,7 @@
 //   m[r]     = max_j R[r, j]
 //   Po[i, j] = max_{r in query group i} exp2(R[r, j] - m[r]);   Po[i, :] /= sum_j Po[i, j]
 //
-// Kernel 1 (MFMA-bound, 2*Ms*Ns*D flops): a dense bf16 contraction of the sampled query rows with the
+// Kernel 1 (MFMA-bound, 2*Ms*Ns*D flops): a dense bf16 / fp16 contraction of the sampled query rows with the
 // sampled key rows, both gathered straight from the un-sampled Q / K through the per-head offset
 // tables.  One workgroup = 4 waves x 64 sampled query rows (two B-operand sets per wave share every K
 // operand read from LDS); the waves share K tiles of 64 sampled keys, copied by global_load_lds into
@@ -25,7 +25,8 @@ constexpr int TK = 64;
 constexpr int EST_MAX_KSPLIT = 4;
 
 struct EstParams {
-  const bf16_t *q, *k;
+  const uint16_t *q, *k;  // bf16 or fp16 (the kernel's element trait says which)
+  int dtype;
   int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl;
   const int32_t *off_q, *off_k;
   const int32_t* q_index;  // optional: the sampled query position i is source row q_index[i] (token re-ordering)
@@ -83,8 +84,9 @@ __device__ __forceinline__ void chunk_max_piece(const f32x16& sc, float (&val)[1
   }
 }
 
-template <int D, int GPC>
+template <int D, int GPC, class ET>
 __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
+  using x8 = typename ET::x8;
   using G = psa_tiles::LtGeom<D>;
   constexpr int KK = D / 16, RS = 2;  // RS sets of 32 query rows per wave
   constexpr int E_TILE = G::TILE, E_ISTR = psa_tiles::LT_ISTR, RPL = G::RPL;
@@ -103,16 +105,16 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
 
   // Q fragments: lane holds Q[row l32 of set rs][16*kk + 8*hh .. +8]
   const int row0 = blockIdx.x * (4 * 32 * RS) + wave * (32 * RS);
-  bf16x8 qf[RS][KK];
+  x8 qf[RS][KK];
   {
     const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * keep_m : nullptr;
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
       int src = sampled_src(row0 + rs * 32 + l32, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
       if (p.q_index != nullptr) src = clamp_row(p.q_index[src], p.Lq);
-      const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
+      const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + hh * 8;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) qf[rs][kk] = *(const bf16x8*)(qp + kk * 16);
+      for (int kk = 0; kk < KK; ++kk) qf[rs][kk] = *(const x8*)(qp + kk * 16);
     }
   }
 
@@ -199,11 +201,11 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
     // step i = chunk c * KK + k-step kk; its operand is requested two steps (four MFMAs) ahead
     auto kread = [&](int i) __attribute__((always_inline)) {
       const int c = i / KK, kk = i % KK;
-      return *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
+      return *(PSA_LDS(const x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
     };
     f32x16 s[RS][2];
     float val[RS][2][NV], tmp[RS][3];
-    bf16x8 ka[3];
+    x8 ka[3];
     ka[0] = kread(0);
     ka[1] = kread(1);
 #pragma unroll
@@ -211,7 +213,7 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
       const int c = i / KK, kk = i % KK;
       if (i + 2 < 2 * KK) ka[(i + 2) % 3] = kread(i + 2);
 #pragma unroll
-      for (int rs = 0; rs < RS; ++rs) s[rs][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[i % 3], qf[rs][kk], kk == 0 ? zero16 : s[rs][c], 0, 0, 0);
+      for (int rs = 0; rs < RS; ++rs) s[rs][c] = ET::mfma(ka[i % 3], qf[rs][kk], kk == 0 ? zero16 : s[rs][c]);
       if (c == 1) {
         __builtin_amdgcn_sched_barrier(0);  // after this step's MFMAs: the first piece waits for chunk 0's last results
 #pragma unroll
@@ -251,6 +253,84 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
 // rows (one contiguous run of the workspace), a wave 256/keep_m key groups per load; the maximum over the
 // group's rows is an in-lane maximum plus a butterfly over those lanes.
 // Leaves the un-normalised row in s_e[0 .. n_d) and returns its sum (fixed summation order); 256 threads.
+// The contraction for fp32 tensors: fp32 operands and arithmetic (vector FMAs), the same workspace contents as the
+// MFMA kernel (group maxima R^T [key group][query row] in log2 units, row maxima; one share of the keys).  One
+// workgroup per 64 sampled query rows; key tiles of 64 sampled keys go to LDS channel-major; thread (t / 16, t % 16)
+// owns rows ty + 16 i and keys tx + 16 j of a tile, the tile's logits pass through LDS for the group maxima.
+template <int D>
+__global__ __launch_bounds__(256) void psa_est_gemm_f32_kernel(EstParams p) {
+  constexpr int DP = D + 1, KP = TK + 1;
+  extern __shared__ __align__(16) unsigned char smem_f32[];
+  float* Qs = (float*)smem_f32;  // [64][DP]
+  float* Kt = Qs + 64 * DP;      // [D][KP]
+  float* Ss = Kt + D * KP;       // [64][KP]
+  const float* qg = (const float*)p.q;
+  const float* kg = (const float*)p.k;
+  const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+  const int bh = blockIdx.y, h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int row0 = blockIdx.x * 64;
+  const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * (1 << p.keep_m_log2) : nullptr;
+  const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * (1 << p.keep_n_log2) : nullptr;
+  for (int u = tid; u < 64 * (D / 4); u += 256) {
+    const int r = u / (D / 4), c4 = u % (D / 4);
+    int src = sampled_src(row0 + r, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
+    if (p.q_index != nullptr) src = clamp_row(p.q_index[src], p.Lq);
+    const f32x4 x = *(const f32x4*)(qg + b * p.q_sb + h * p.q_sh + (int64_t)src * p.q_sl + c4 * 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) Qs[r * DP + c4 * 4 + e] = x[e];
+  }
+  const int keep_n = 1 << p.keep_n_log2, gpt = TK >> p.keep_n_log2;  // key groups per tile
+  float m_run = -INFINITY;  // of row (tid / 4) for the threads that write group maxima, see below
+  float* rt = p.rt + (int64_t)bh * p.n_d * p.Ms_pad + row0;
+  const float* kb = kg + b * p.k_sb + hk * p.k_sh;
+  for (int t0 = 0; t0 < p.Ns_pad; t0 += TK) {
+    __syncthreads();
+    for (int u = tid; u < TK * (D / 4); u += 256) {
+      const int r = u / (D / 4), c4 = u % (D / 4);
+      const int src = sampled_src(t0 + r, p.Ns, p.keep_n_log2, p.bn, ok, p.Lk);
+      const f32x4 x = *(const f32x4*)(kb + (int64_t)src * p.k_sl + c4 * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) Kt[(c4 * 4 + e) * KP + r] = x[e];
+    }
+    __syncthreads();
+    float s[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[i][j] = 0.f;
+    for (int d = 0; d < D; ++d) {
+      float qv[4], kv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) qv[i] = Qs[(ty + 16 * i) * DP + d];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kv[j] = Kt[d * KP + tx + 16 * j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[i][j] = __builtin_fmaf(qv[i], kv[j], s[i][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) Ss[(ty + 16 * i) * KP + tx + 16 * j] = s[i][j] * p.qk_scale;
+    __syncthreads();
+    // group maxima: (row, group) pairs, row fastest so that the stores are coalesced
+    for (int u = tid; u < 64 * gpt; u += 256) {
+      const int r = u & 63, g = u >> 6;
+      float mx = -INFINITY;
+      for (int c = 0; c < keep_n; ++c) mx = fmaxf(mx, Ss[r * KP + g * keep_n + c]);
+      rt[(int64_t)((t0 >> p.keep_n_log2) + g) * p.Ms_pad + r] = mx;
+    }
+    // row maxima: thread t < 64 keeps the maximum of row t
+    if (tid < 64) {
+      float mx = m_run;
+      for (int c = 0; c < TK; ++c) mx = fmaxf(mx, Ss[tid * KP + c]);
+      m_run = mx;
+    }
+  }
+  if (tid < 64) p.mrow[(int64_t)bh * p.Ms_pad + row0 + tid] = m_run;
+}
+
 __device__ __forceinline__ float est_reduce_row(const EstParams& p, float* s_e, float* s_part, int i, int bh) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lpg_log2 = p.keep_m_log2 - 2;            // lanes per key group
@@ -326,11 +406,21 @@ int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp
   const int tiles = p.Ns_pad / TK;
   while (p.ksplit < EST_MAX_KSPLIT && wgs * p.ksplit < 3 * 256 && tiles / (p.ksplit * 2) >= 8) p.ksplit *= 2;
   grid.z = (unsigned)p.ksplit;
-  switch (p.keep_n_log2) {
-    case 5: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 0>), grid, dim3(256), 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 1>), grid, dim3(256), 0, stream, p); break;
-    default: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 2>), grid, dim3(256), 0, stream, p); break;
+  if (p.dtype == PSA_DTYPE_F32) {
+    p.ksplit = 1;
+    const size_t shmem = (size_t)(64 * (D + 1) + D * (TK + 1) + 64 * (TK + 1)) * sizeof(float);
+    if (hipFuncSetAttribute((const void*)psa_est_gemm_f32_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+      return PSA_ERR_LAUNCH;
+    hipLaunchKernelGGL(psa_est_gemm_f32_kernel<D>, dim3((unsigned)(p.Ms_pad / 64), (unsigned)(B * p.Hq)), dim3(256), shmem, stream, p);
   }
+  psa_dispatch16(p.dtype, [&](auto et) {
+    using ET = decltype(et);
+    switch (p.keep_n_log2) {
+      case 5: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 0, ET>), grid, dim3(256), 0, stream, p); break;
+      case 4: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 1, ET>), grid, dim3(256), 0, stream, p); break;
+      default: hipLaunchKernelGGL((psa_est_gemm_lds_kernel<D, 2, ET>), grid, dim3(256), 0, stream, p); break;
+    }
+  });
   const int rc = psa_check_launch("psa_estimate_sampled (contraction)");
   if (rc != PSA_OK) return rc;
   const dim3 rgrid((unsigned)p.out_rows, (unsigned)(B * p.Hq));
@@ -389,6 +479,9 @@ int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* o
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Lq > 0 && Lk > 0, PSA_ERR_ARG, "psa_estimate_sampled: sizes must be positive");
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_estimate_sampled: Hq must be a multiple of Hkv");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: B*Hq too large");
+  PSA_REQUIRE(q.dtype == k.dtype, PSA_ERR_ARG, "psa_estimate_sampled: q and k must share one element type");
+  PSA_REQUIRE(q.dtype == PSA_DTYPE_BF16 || q.dtype == PSA_DTYPE_F16 || q.dtype == PSA_DTYPE_F32, PSA_ERR_ARG,
+              "psa_estimate_sampled: unknown element type %d", q.dtype);
   PSA_REQUIRE(D == 64 || D == 128, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: head dim %d not in {64, 128}", D);
   PSA_REQUIRE(keep_m == 8 || keep_m == 16 || keep_m == 32, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: keep_m=%d not in {8,16,32}", keep_m);
   PSA_REQUIRE(keep_n == 8 || keep_n == 16 || keep_n == 32, PSA_ERR_UNSUPPORTED, "psa_estimate_sampled: keep_n=%d not in {8,16,32}", keep_n);
@@ -400,7 +493,7 @@ int est_run(psa_tensor4 q, psa_tensor4 k, const int32_t* off_q, const int32_t* o
               "psa_estimate_sampled: one (batch, head) slice of K must span less than 4 GiB");
   const EstGeom g = est_geom(Lq, Lk, block_m, block_n, keep_m, keep_n);
   EstParams p;
-  p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr;
+  p.q = (const uint16_t*)q.ptr; p.k = (const uint16_t*)k.ptr; p.dtype = q.dtype;
   p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sl = q.stride_l;
   p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sl = k.stride_l;
   p.off_q = off_q; p.off_k = off_k; p.q_index = q_index; p.scores = scores;

@@ -36,6 +36,11 @@
 #include "psa_order.h"
 #include "psa_schedule.h"
 
+// fp32 tensors: psa_f32.hip
+int psa_fwd_f32(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool, const void* v_pool, const void* map, int map_elem_bytes,
+                psa_tensor4 out, float* lse, int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, float sm_scale, int causal,
+                psa_stream_t stream, const int32_t* q_index);
+
 namespace {
 
 #ifndef PSA_FWD_ONE_GROUP
@@ -57,12 +62,12 @@ __device__ __forceinline__ void static_for(F&& f) {
 constexpr float LAZY_THRESHOLD = 8.f;  // log2 units the running max may lag behind
 
 struct FwdParams {
-  const bf16_t *q, *k, *v;
+  const uint16_t *q, *k, *v;  // bf16 or fp16: the kernel's element trait says which
   int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, o_sb, o_sh, o_sl;
-  const bf16_t *kp, *vp;  // pooled levels 2,4,8 (may be null when map is null)
+  const uint16_t *kp, *vp;  // pooled levels 2,4,8 (may be null when map is null)
   const void* map;
   int map_elem;
-  bf16_t* o;
+  uint16_t* o;
   float* lse;
   int B, Hq, Hkv, L, Mq, Nk, bn_log2, bm;
   int64_t npad;
@@ -73,6 +78,7 @@ struct FwdParams {
   int grp_bytes;  // two-group kernel: LDS bytes of one group (tile buffers + schedule)
   const int32_t* order;  // optional: logical workgroup id -> (b, h, q-block) row, longest rows first per XCD
   const int32_t* q_index;  // optional (token re-ordering): query / output position i lives in row q_index[i] of q, out, lse
+  int dtype;               // PSA_DTYPE_BF16 / PSA_DTYPE_F16
   // prebuilt tile schedule (psa_schedule.h), scheduled kernel only: tiles per row and the rows' tile records
   const u32x4* sched_rec;
   const int32_t* sched_tiles;
@@ -88,8 +94,9 @@ constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the blocks of a til
     __syncthreads();                        \
   } while (0)
 
-template <int D, int NW>
+template <int D, int NW, class ET>
 __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
+  using x8 = typename ET::x8;
   using G = psa_tiles::LtGeom<D>;
   constexpr int F_TILE = G::TILE;  // bytes of one K or V tile
   constexpr int NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
@@ -132,13 +139,13 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   // Q fragments (B operand of S^T = K Q^T): lane holds Q[row l32][16*kk + 8*hh .. +8]
   const int q_row0 = I * BM + wave * 32;
   const int q_idx = q_row0 + l32;
-  bf16x8 qf[KK];
+  x8 qf[KK];
   {
     int qr = q_idx < P_L ? q_idx : P_L - 1;
     if (p.q_index != nullptr) qr = clamp_row(p.q_index[qr], P_L);
-    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+    const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const x8*)(qp + kk * 16);
   }
   const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2,
                                                  P_L, P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
@@ -170,7 +177,6 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
   float m_run = -INFINITY;  // running reference max (log2 domain), same in both half-waves
   float l_run = 0.f;        // this lane's partial row sum
-  const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
 
   // masks (if needed) and reduces the logits of tile t; returns the bias - reference max and the rescale factor
   auto softmax_head = [&](int t, f32x16 (&s_cur)[2], float& nb, float& alpha) __attribute__((always_inline)) {
@@ -226,8 +232,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
     for (int e = 0; e < 4; e += 2) {
       const float p0 = fast_exp2(__builtin_fmaf(sc[i + e], P_scale_log2, nb));
       const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb));
-      pk2[e >> 1] = pack_bf16x2(p0, p1);
-      lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk2[e >> 1]), ones, lsum, false);
+      pk2[e >> 1] = ET::pack2(p0, p1);
+      lsum = ET::add_pair(pk2[e >> 1], lsum);
     }
   };
   // exponentials of the 16 logits of one 32-key half (4 groups of 4)
@@ -243,16 +249,16 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s2[c][i] = 0.f;
-    bf16x8 a0 = *(PSA_LDS(const bf16x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const bf16x8))(Ks + k_off[0] + G::HALF);
+    x8 a0 = *(PSA_LDS(const x8))(Ks + k_off[0]), a1 = *(PSA_LDS(const x8))(Ks + k_off[0] + G::HALF);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      bf16x8 n0 = a0, n1 = a1;
+      x8 n0 = a0, n1 = a1;
       if (kk + 1 < KK) {
-        n0 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
-        n1 = *(PSA_LDS(const bf16x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + G::HALF);
+        n0 = *(PSA_LDS(const x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64);
+        n1 = *(PSA_LDS(const x8))(Ks + k_off[(kk + 1) & 1] + ((kk + 1) >> 1) * 64 + G::HALF);
       }
-      s2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[kk], s2[0], 0, 0, 0);
-      s2[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[kk], s2[1], 0, 0, 0);
+      s2[0] = ET::mfma(a0, qf[kk], s2[0]);
+      s2[1] = ET::mfma(a1, qf[kk], s2[1]);
       a0 = n0;
       a1 = n1;
     }
@@ -265,8 +271,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
     // operand of MFMA step st = DB*g + db; reads run AHEAD steps in front of the MFMAs
     constexpr int AHEAD = 2, STEPS = 2 * DB;
     auto vread = [&](int st, int s) __attribute__((always_inline)) {
-      return __builtin_bit_cast(
-          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[s] + (st % DB) * 64 + (st / DB) * G::GROUP)));
+      return ET::read_tr(Vs + v_off[s] + (st % DB) * 64 + (st / DB) * G::GROUP);
     };
     u32x2 vlo[STEPS], vhi[STEPS];  // fully unrolled: every element is a short-lived register value
 #pragma unroll
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
       }
       u32x4 bw = {pk8[g * 4 + 0], pk8[g * 4 + 1], pk8[g * 4 + 2], pk8[g * 4 + 3]};
       u32x4 aw = {vlo[st][0], vlo[st][1], vhi[st][0], vhi[st][1]};
-      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), __builtin_bit_cast(bf16x8, bw), acc[db], 0, 0, 0);
+      acc[db] = ET::mfma(__builtin_bit_cast(x8, aw), __builtin_bit_cast(x8, bw), acc[db]);
       __builtin_amdgcn_sched_barrier(0);  // keep the reads AHEAD steps in front, not more
     }
   };
@@ -349,12 +354,12 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
-      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
-      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
+      w[0] = ET::pack2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
+      w[1] = ET::pack2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
       *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
     }
   __syncthreads();
-  bf16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
+  uint16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
   for (int u = tid; u < BM * CH; u += NT) {
     const int r = u / CH, ch = u % CH;
     const int row = I * BM + r;
@@ -390,8 +395,9 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
 // two instructions (M0, then the load with the row step n * 256 as its immediate offset - which the hardware also adds
 // on the LDS side, so M0 carries the difference), the base pointer of a tile's level is kept while the level stays the
 // same (tiles of a row are sorted by level), and nothing is looked up per lane.
-template <int D, int NW, bool GS>
+template <int D, int NW, bool GS, class ET>
 __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p) {
+  using x8 = typename ET::x8;
   using G = psa_tiles::LtGeom<D>;
   constexpr int F_TILE = G::TILE;
   constexpr int NT = NW * 64, BM = NW * 32, KK = D / 16, DB = D / 32, CH = D / 8;
@@ -438,13 +444,13 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
   if (!active) jmax = 0;
   const int q_row0 = I * BM + wave * 32;
   const int q_idx = q_row0 + l32;
-  bf16x8 qf[KK];
+  x8 qf[KK];
   {
     int qr = q_idx < P_L ? q_idx : P_L - 1;
     if (p.q_index != nullptr) qr = clamp_row(p.q_index[qr], P_L);
-    const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
+    const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 16);
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const x8*)(qp + kk * 16);
   }
   // the row's tile records (GS): read through the scalar cache; wp walks this wave's word of the records
   using w_ptr = const __attribute__((address_space(4))) uint32_t*;
@@ -581,7 +587,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     for (int e = 0; e < 4; e += 2) {
       const float p0 = fast_exp2(e == 0 ? x0 : __builtin_fmaf(sc[i + e], P_scale_log2, nb_));
       const float p1 = fast_exp2(__builtin_fmaf(sc[i + e + 1], P_scale_log2, nb_));
-      pk2[e >> 1] = pack_bf16x2(p0, p1);
+      pk2[e >> 1] = ET::pack2(p0, p1);
       lsum += p0 + p1;
     }
   };
@@ -596,7 +602,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     int row[G::RPL];
   };
   // base pointers of the pooled levels of this (batch, kv head); plain scalars, selected by compare chains
-  auto pool_base = [&](const bf16_t* pool, int lv) __attribute__((always_inline)) {
+  auto pool_base = [&](const uint16_t* pool, int lv) __attribute__((always_inline)) {
     return (const char*)pool + (BHkv * (P_npad - (P_npad >> (lv - 1))) + bhk * (P_npad >> lv)) * (D * 2);
   };
   const char* const kb1 = pool_base(P_kp, 1);
@@ -631,10 +637,10 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     PSA_LDS(unsigned char) Vs = (PSA_LDS(unsigned char))(smem_all) + (2 + (KB ^ 1)) * F_TILE;
     constexpr int K_UP = KK - 2;          // k-steps whose K operands are requested before the first MFMA
     constexpr int V_LATE = 2 * (KK - K_UP);  // PV steps whose operands are requested during PV
-    bf16x8 ka[2 * KK];
+    x8 ka[2 * KK];
     auto kread = [&](int kk) __attribute__((always_inline)) {
-      ka[2 * kk] = *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64);
-      ka[2 * kk + 1] = *(PSA_LDS(const bf16x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + G::HALF);
+      ka[2 * kk] = *(PSA_LDS(const x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64);
+      ka[2 * kk + 1] = *(PSA_LDS(const x8))(Ks + k_off[kk & 1] + (kk >> 1) * 64 + G::HALF);
     };
 #pragma unroll
     for (int kk = 0; kk < K_UP; ++kk) kread(kk);
@@ -647,13 +653,13 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
     auto vread = [&](int st) __attribute__((always_inline)) {
       const int cg = st / DB, db = st % DB;
       const int off = (cg >> 1) * G::HALF + db * 64 + (cg & 1) * G::GROUP;
-      vlo[st] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[0] + off)));
-      vhi[st] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Vs + v_off[1] + off)));
+      vlo[st] = ET::read_tr(Vs + v_off[0] + off);
+      vhi[st] = ET::read_tr(Vs + v_off[1] + off);
     };
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      s2[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[2 * kk], qf[kk], s2[0], 0, 0, 0);
-      s2[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[2 * kk + 1], qf[kk], s2[1], 0, 0, 0);
+      s2[0] = ET::mfma(ka[2 * kk], qf[kk], s2[0]);
+      s2[1] = ET::mfma(ka[2 * kk + 1], qf[kk], s2[1]);
       if (kk + K_UP < KK) {
         kread(kk + K_UP);
       } else {
@@ -676,7 +682,7 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
       const int g = cg & 1;
       u32x4 bw = {pk8[g * 4 + 0], pk8[g * 4 + 1], pk8[g * 4 + 2], pk8[g * 4 + 3]};
       u32x4 aw = {vlo[st][0], vlo[st][1], vhi[st][0], vhi[st][1]};
-      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), __builtin_bit_cast(bf16x8, bw), acc[db], 0, 0, 0);
+      acc[db] = ET::mfma(__builtin_bit_cast(x8, aw), __builtin_bit_cast(x8, bw), acc[db]);
       if (st < V_LATE) vread(STEPS - V_LATE + st);
       hook(st);
       __builtin_amdgcn_sched_barrier(0);
@@ -929,13 +935,13 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
-      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
-      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
+      w[0] = ET::pack2(acc[db][g * 4 + 0] * inv, acc[db][g * 4 + 1] * inv);
+      w[1] = ET::pack2(acc[db][g * 4 + 2] * inv, acc[db][g * 4 + 3] * inv);
       *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
     }
   __syncthreads();
   if (active) {
-    bf16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
+    uint16_t* ob = p.o + b * p.o_sb + h * p.o_sh;
     for (int u = tid; u < BM * CH; u += NT) {
       const int r = u / CH, ch = u % CH;
       const int row = I * BM + r;
@@ -952,10 +958,16 @@ template <int D, int NW>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
   size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
   if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-  if (hipFuncSetAttribute((const void*)psa_fwd_lds_kernel<D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-    return PSA_ERR_LAUNCH;
-  hipLaunchKernelGGL((psa_fwd_lds_kernel<D, NW>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
-  return PSA_OK;
+  int rc = PSA_OK;
+  psa_dispatch16(p.dtype, [&](auto et) {
+    using ET = decltype(et);
+    if (hipFuncSetAttribute((const void*)psa_fwd_lds_kernel<D, NW, ET>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) {
+      rc = PSA_ERR_LAUNCH;
+      return;
+    }
+    hipLaunchKernelGGL((psa_fwd_lds_kernel<D, NW, ET>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
+  });
+  return rc;
 }
 
 template <int D, int NW, bool GS>
@@ -964,10 +976,16 @@ int launch_fwd_pp(FwdParams& p, int Nk, hipStream_t stream) {
   const size_t sched = GS ? 0 : ((((size_t)p.max_tiles * 8 + (size_t)Nk * 2) + 15) & ~(size_t)15);
   p.grp_bytes = (int)(4 * psa_tiles::LtGeom<D>::TILE + sched);
   const size_t shmem = 2 * (size_t)p.grp_bytes;
-  if (hipFuncSetAttribute((const void*)psa_fwd_pp_kernel<D, NW, GS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-    return PSA_ERR_LAUNCH;
-  hipLaunchKernelGGL((psa_fwd_pp_kernel<D, NW, GS>), dim3((unsigned)((p.wg_chunk / 2) * p.wg_groups)), dim3(2 * NW * 64), shmem, stream, p);
-  return PSA_OK;
+  int rc = PSA_OK;
+  psa_dispatch16(p.dtype, [&](auto et) {
+    using ET = decltype(et);
+    if (hipFuncSetAttribute((const void*)psa_fwd_pp_kernel<D, NW, GS, ET>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) {
+      rc = PSA_ERR_LAUNCH;
+      return;
+    }
+    hipLaunchKernelGGL((psa_fwd_pp_kernel<D, NW, GS, ET>), dim3((unsigned)((p.wg_chunk / 2) * p.wg_groups)), dim3(2 * NW * 64), shmem, stream, p);
+  });
+  return rc;
 }
 // LDS bytes the two-group kernel needs (tile buffers and schedule of both groups + its static tables)
 template <int D>
@@ -992,6 +1010,10 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
   PSA_REQUIRE(map == nullptr || (k_pool && v_pool), PSA_ERR_ARG, "psa_fwd: pooled K/V required with a level map");
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_fwd: map_elem_bytes must be 1 or 4");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0, PSA_ERR_ARG, "psa_fwd: B, H, L must be positive");
+  PSA_REQUIRE(q.dtype == k.dtype && q.dtype == v.dtype && q.dtype == out.dtype, PSA_ERR_ARG, "psa_fwd: q, k, v, out must share one element type");
+  if (q.dtype == PSA_DTYPE_F32)
+    return psa_fwd_f32(q, k, v, k_pool, v_pool, map, map_elem_bytes, out, lse, B, Hq, Hkv, L, D, block_m, block_n, sm_scale, causal, stream, q_index);
+  PSA_REQUIRE(q.dtype == PSA_DTYPE_BF16 || q.dtype == PSA_DTYPE_F16, PSA_ERR_ARG, "psa_fwd: unknown element type %d", q.dtype);
   PSA_REQUIRE(Hq % Hkv == 0, PSA_ERR_ARG, "psa_fwd: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
   PSA_REQUIRE(sm_scale > 0.f, PSA_ERR_ARG, "psa_fwd: sm_scale must be positive");
   PSA_REQUIRE(D == 64 || D == 128, PSA_ERR_UNSUPPORTED, "psa_fwd: head dim %d not in {64, 128}", D);
@@ -1008,13 +1030,13 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
   const int64_t total = (int64_t)B * Hq * Mq;
   PSA_REQUIRE(total < (1ll << 28), PSA_ERR_UNSUPPORTED, "psa_fwd: too many workgroups");
   FwdParams p;
-  p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr; p.v = (const bf16_t*)v.ptr; p.o = (bf16_t*)out.ptr;
+  p.q = (const uint16_t*)q.ptr; p.k = (const uint16_t*)k.ptr; p.v = (const uint16_t*)v.ptr; p.o = (uint16_t*)out.ptr;
   p.q_sb = q.stride_b; p.q_sh = q.stride_h; p.q_sl = q.stride_l;
   p.k_sb = k.stride_b; p.k_sh = k.stride_h; p.k_sl = k.stride_l;
   p.v_sb = v.stride_b; p.v_sh = v.stride_h; p.v_sl = v.stride_l;
   p.o_sb = out.stride_b; p.o_sh = out.stride_h; p.o_sl = out.stride_l;
-  p.kp = (const bf16_t*)k_pool; p.vp = (const bf16_t*)v_pool;
-  p.map = map; p.map_elem = map_elem_bytes; p.lse = lse;
+  p.kp = (const uint16_t*)k_pool; p.vp = (const uint16_t*)v_pool;
+  p.map = map; p.map_elem = map_elem_bytes; p.lse = lse; p.dtype = q.dtype;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.L = L; p.Mq = Mq; p.Nk = Nk;
   p.bn_log2 = psa_ilog2(block_n); p.bm = block_m;
   p.npad = (int64_t)Nk * block_n;

@@ -10,19 +10,20 @@
 namespace {
 
 struct KsimParams {
-  const bf16_t* k;
+  const uint16_t* k;  // bf16 or fp16
   int64_t sb, sh, sl;
   int32_t* out;
   int H, L, D, bn, Nk;
   float t2, t4, t8;
 };
 
+template <class ET>
 __global__ __launch_bounds__(256) void psa_ksim_kernel(KsimParams p) {
   __shared__ float s_part[3][16];
   const int lpr = p.D >> 3;
   const int J = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
   const int g = threadIdx.x / lpr, c = threadIdx.x % lpr;
-  const bf16_t* src = p.k + b * p.sb + h * p.sh + c * 8;
+  const uint16_t* src = p.k + b * p.sb + h * p.sh + c * 8;
   float f[8][8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -31,8 +32,8 @@ __global__ __launch_bounds__(256) void psa_ksim_kernel(KsimParams p) {
     const u32x4 w = *(const u32x4*)(src + row * p.sl);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      f[i][2 * j] = bf16_bits_to_f32(w[j] & 0xffffu);
-      f[i][2 * j + 1] = __builtin_bit_cast(float, w[j] & 0xffff0000u);
+      f[i][2 * j] = ET::from_bits(w[j] & 0xffffu);
+      f[i][2 * j + 1] = ET::from_bits(w[j] >> 16);
     }
   }
   // 8 squared norms, dots (0,1) (2,3) (4,5) (6,7) | (0,3) (4,7) | (0,7)
@@ -96,10 +97,13 @@ extern "C" int psa_ksim(psa_tensor4 k, int32_t* cap_out, int B, int H, int L, in
   PSA_REQUIRE(((uintptr_t)k.ptr % 16 == 0) && k.stride_b % 8 == 0 && k.stride_h % 8 == 0 && k.stride_l % 8 == 0, PSA_ERR_UNSUPPORTED,
               "psa_ksim: K must be 16-byte aligned with strides that are multiples of 8 elements");
   KsimParams p;
-  p.k = (const bf16_t*)k.ptr; p.sb = k.stride_b; p.sh = k.stride_h; p.sl = k.stride_l;
+  p.k = (const uint16_t*)k.ptr; p.sb = k.stride_b; p.sh = k.stride_h; p.sl = k.stride_l;
   p.out = cap_out; p.H = H; p.L = L; p.D = D; p.bn = block_n; p.Nk = (L + block_n - 1) / block_n;
   p.t2 = thr2; p.t4 = thr4; p.t8 = thr8;
-  hipLaunchKernelGGL(psa_ksim_kernel, dim3((unsigned)p.Nk, (unsigned)(B * H)), dim3((unsigned)((block_n / 8) * (D / 8))), 0,
-                     (hipStream_t)stream, p);
+  const bool known = psa_dispatch16(k.dtype, [&](auto et) {
+    hipLaunchKernelGGL(psa_ksim_kernel<decltype(et)>, dim3((unsigned)p.Nk, (unsigned)(B * H)), dim3((unsigned)((block_n / 8) * (D / 8))), 0,
+                       (hipStream_t)stream, p);
+  });
+  PSA_REQUIRE(known, PSA_ERR_UNSUPPORTED, "psa_ksim: bf16 or fp16 keys only");
   return psa_check_launch("psa_ksim");
 }

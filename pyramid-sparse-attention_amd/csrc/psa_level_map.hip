@@ -172,6 +172,78 @@ extern "C" int psa_map_from_list(const int32_t* list, void* map_out, int map_ele
 }
 
 // ---------------------------------------------------------------------------------------
+// dense map -> index list (five segments: levels 1, 2, 4, 8, then the skipped blocks; -1 after each)
+// ---------------------------------------------------------------------------------------
+// One wave per row.  Blocks are listed by level, ascending inside a level; a segment's length is rounded down to a
+// multiple of ceil(level / align_div) and the blocks that do not fit lead the next segment.
+__global__ __launch_bounds__(256) void psa_list_from_map_kernel(const void* map, int map_elem, int32_t* list, int64_t rows, int Nk,
+                                                              int align_div) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t mrow = row * Nk;
+  int32_t* out = list + row * (Nk + 5);
+  // segment of a level value: 1, 2, 4, 8 -> 0..3, anything else (0 = skipped) -> 4
+  auto seg_of = [](int lvl) { return lvl == 1 ? 0 : lvl == 2 ? 1 : lvl == 4 ? 2 : lvl == 8 ? 3 : 4; };
+  int cnt[5] = {0, 0, 0, 0, 0};
+  for (int j0 = 0; j0 < Nk; j0 += 64) {
+    const int j = j0 + lane;
+    const int sg = j < Nk ? seg_of(load_map(map, mrow + j, map_elem)) : -1;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) cnt[t] += __popcll(__ballot(sg == t));
+  }
+  int start[5], bound[5];  // first sorted position of a level; end of a segment after the rounding
+  {
+    int a = 0;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) {
+      start[t] = a;
+      a += cnt[t];
+    }
+    int carry = 0, b = 0;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) {
+      int len = cnt[t] + carry;
+      carry = 0;
+      if (t < 4) {
+        const int mult = ((1 << t) + align_div - 1) / align_div;
+        carry = mult > 1 ? len % mult : 0;
+        len -= carry;
+      }
+      b += len;
+      bound[t] = b;
+    }
+  }
+  if (lane < 5) out[bound[lane] + lane] = -1;  // the separator behind segment `lane`
+  int run[5] = {start[0], start[1], start[2], start[3], start[4]};
+  const uint64_t lt_mask = (1ull << lane) - 1ull;
+  for (int j0 = 0; j0 < Nk; j0 += 64) {
+    const int j = j0 + lane;
+    const int sg = j < Nk ? seg_of(load_map(map, mrow + j, map_elem)) : -1;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) {
+      const uint64_t bal = __ballot(sg == t);
+      if (sg == t) {
+        const int pos = run[t] + __popcll(bal & lt_mask);  // position in the list sorted by level
+        const int seps = (pos >= bound[0]) + (pos >= bound[1]) + (pos >= bound[2]) + (pos >= bound[3]) + (pos >= bound[4]);
+        out[pos + seps] = j;
+      }
+      run[t] += __popcll(bal);
+    }
+  }
+}
+
+extern "C" int psa_list_from_map(const void* map, int map_elem_bytes, int32_t* list_out, int64_t rows, int Nk, int align_div,
+                                 psa_stream_t stream) {
+  PSA_REQUIRE(map && list_out, PSA_ERR_ARG, "psa_list_from_map: null pointer");
+  PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_list_from_map: map_elem_bytes must be 1 or 4");
+  PSA_REQUIRE(rows > 0 && rows < (1ll << 31) && Nk > 0 && align_div >= 1, PSA_ERR_ARG, "psa_list_from_map: bad sizes");
+  hipLaunchKernelGGL(psa_list_from_map_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, map,
+                     map_elem_bytes, list_out, rows, Nk, align_div);
+  return psa_check_launch("psa_list_from_map");
+}
+
+// ---------------------------------------------------------------------------------------
 // map = min(map, cap[bh, col])
 // ---------------------------------------------------------------------------------------
 __global__ void psa_map_min_cap_kernel(void* map, int map_elem, const int32_t* cap, int Mq, int Nk) {

@@ -19,8 +19,12 @@ PSA_MODE_THRESHOLDBOUND = 1
 PSA_MAX_LEVEL_ITEMS = 8
 
 
+PSA_DTYPE_BF16, PSA_DTYPE_F16, PSA_DTYPE_F32 = 0, 1, 2
+
+
 class Tensor4(Structure):
-    _fields_ = [("ptr", c_void_p), ("stride_b", c_int64), ("stride_h", c_int64), ("stride_l", c_int64)]
+    _fields_ = [("ptr", c_void_p), ("stride_b", c_int64), ("stride_h", c_int64), ("stride_l", c_int64), ("dtype", c_int32),
+                ("reserved", c_int32)]
 
 
 # name -> (restype, argtypes); one entry per symbol declared in include/psa_hip.h
@@ -59,6 +63,7 @@ SIGNATURES = {
         [Tensor4, Tensor4, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     ),
     "psa_map_from_list": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_void_p]),
+    "psa_list_from_map": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "psa_ksim": (c_int, [Tensor4, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p]),
     "psa_map_min_cap": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "psa_density": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),

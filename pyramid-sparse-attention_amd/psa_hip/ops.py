@@ -21,18 +21,38 @@ def _require_gpu(*ts):
             raise RuntimeError("psa_hip operators run on the GPU only (got a %s tensor); there is no CPU path" % t.device)
 
 
-def _bf16_view(x: torch.Tensor) -> torch.Tensor:
-    """[B,H,L,D] tensor usable by the kernels: bf16, D contiguous, 16-byte aligned rows."""
+_DTYPE_ID = {torch.bfloat16: _lib.PSA_DTYPE_BF16, torch.float16: _lib.PSA_DTYPE_F16, torch.float32: _lib.PSA_DTYPE_F32}
+
+
+def _kernel_view(x: torch.Tensor, types=(torch.bfloat16, torch.float16, torch.float32)) -> torch.Tensor:
+    """[B,H,L,D] tensor usable by the kernels: one of `types` (the element types the operator has kernels for: the
+    tensor is computed on in its own type; any other type is rounded to bf16 first), D contiguous, 16-byte aligned
+    rows."""
     if x.dim() != 4:
         raise ValueError("expected a [B, H, L, D] tensor, got shape %s" % (tuple(x.shape),))
-    if x.dtype != torch.bfloat16:
+    if x.dtype not in types:
         x = x.to(torch.bfloat16)
-    ok = x.stride(3) == 1 and all(s % 8 == 0 for s in x.stride()[:3]) and x.data_ptr() % 16 == 0
+    per16 = 16 // x.element_size()
+    ok = x.stride(3) == 1 and all(s % per16 == 0 for s in x.stride()[:3]) and x.data_ptr() % 16 == 0
     return x if ok else x.contiguous()
 
 
+def _bf16_view(x: torch.Tensor) -> torch.Tensor:
+    """For the operators whose kernels take bf16 only (backward, antidiagonal estimate)."""
+    return _kernel_view(x, (torch.bfloat16,))
+
+
+_T16 = (torch.bfloat16, torch.float16)
+
+
+def _same_type(*ts):
+    """Tensors of one call share one element type: anything that differs from the first is converted to it."""
+    dt = ts[0].dtype
+    return tuple(t if t.dtype == dt else t.to(dt) for t in ts)
+
+
 def _t4(x: torch.Tensor) -> Tensor4:
-    return Tensor4(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2))
+    return Tensor4(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), _DTYPE_ID[x.dtype], 0)
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -45,19 +65,19 @@ def pool_kv(k: torch.Tensor, v: torch.Tensor, block_n: int, out: Optional[Tuple[
     """One pass over K and V -> flat pooled buffers holding levels 2, 4, 8 (see pool_levels).  out: the two buffers,
     allocated by the caller (bf16, psa_pool_elems elements each)."""
     _require_gpu(k, v)
-    k, v = _bf16_view(k), _bf16_view(v)
+    k, v = _same_type(_kernel_view(k), _kernel_view(v))
     B, H, L, D = k.shape
     if v.shape != k.shape:
         raise ValueError("k and v must have the same shape")
     n = lib.psa_pool_elems(B, H, L, D, block_n)
     if out is None:
-        kp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
-        vp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+        kp = torch.empty(n, dtype=k.dtype, device=k.device)
+        vp = torch.empty(n, dtype=k.dtype, device=k.device)
     else:
         kp, vp = out
         for t in (kp, vp):
-            if t.dtype != torch.bfloat16 or t.numel() != n or not t.is_contiguous() or t.device != k.device:
-                raise ValueError("pool_kv: out must be two contiguous bf16 buffers of %d elements on %s" % (n, k.device))
+            if t.dtype != k.dtype or t.numel() != n or not t.is_contiguous() or t.device != k.device:
+                raise ValueError("pool_kv: out must be two contiguous %s buffers of %d elements on %s" % (k.dtype, n, k.device))
     with torch.cuda.device(k.device):
         check(lib.psa_pool_kv(_t4(k), _t4(v), _ptr(kp), _ptr(vp), B, H, L, D, block_n, _stream(k)), "psa_pool_kv")
     return kp, vp
@@ -102,14 +122,14 @@ def pool_kv_indexed(k: torch.Tensor, v: torch.Tensor, index: torch.Tensor, block
     """pool_kv of the re-ordered K, V (position i = source row index[i]; index an int32 permutation of 0..L-1) without a
     gather pass of its own: returns (k_pool, v_pool, k_ord, v_ord), the last two being the re-ordered rows [B,H,L,D]."""
     _require_gpu(k, v, index)
-    k, v = _bf16_view(k), _bf16_view(v)
+    k, v = _same_type(_kernel_view(k), _kernel_view(v))
     B, H, L, D = k.shape
     if v.shape != k.shape:
         raise ValueError("k and v must have the same shape")
     index = _check_index(index, L)
     n = lib.psa_pool_elems(B, H, L, D, block_n)
-    kp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
-    vp = torch.empty(n, dtype=torch.bfloat16, device=k.device)
+    kp = torch.empty(n, dtype=k.dtype, device=k.device)
+    vp = torch.empty(n, dtype=k.dtype, device=k.device)
     ko, vo = torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
     with torch.cuda.device(k.device):
         check(lib.psa_pool_kv_indexed(_t4(k), _t4(v), _ptr(index), _t4(ko), _t4(vo), _ptr(kp), _ptr(vp), B, H, L, D, block_n,
@@ -169,7 +189,7 @@ def estimate_sampled(
     (None: rows are taken as 0..keep-1 of each block).  q_index (int32 permutation [Lq]): query position i is row
     q_index[i] of q (token re-ordering read on the fly; k is passed already re-ordered)."""
     _require_gpu(q, k, off_q, off_k, q_index)
-    q, k = _bf16_view(q), _bf16_view(k)
+    q, k = _same_type(_kernel_view(q), _kernel_view(k))
     B, Hq, Lq, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
     sm_scale = D ** -0.5 if sm_scale is None else sm_scale
@@ -220,7 +240,7 @@ def estimate_sampled_map(
     if map_dtype not in (torch.int8, torch.int32):
         raise ValueError("map_dtype must be int8 or int32")
     _require_gpu(q, k, off_q, off_k, q_index)
-    q, k = _bf16_view(q), _bf16_view(k)
+    q, k = _same_type(_kernel_view(q), _kernel_view(k))
     B, Hq, Lq, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
     sm_scale = D ** -0.5 if sm_scale is None else sm_scale
@@ -390,10 +410,24 @@ def map_from_list(list_mask: torch.Tensor, Nk: int, map_dtype: torch.dtype = tor
     return out
 
 
+def list_from_map(level_map_: torch.Tensor, blocksize: int = 32, compute_tile: int = 32) -> torch.Tensor:
+    """Dense level map [..., Nk] (int8 / int32) -> index list [..., Nk + 5] int32 (levels 1, 2, 4, 8, skipped; -1 behind
+    each segment; segment lengths rounded down to the level's alignment)."""
+    _require_gpu(level_map_)
+    m = level_map_ if level_map_.dtype in (torch.int8, torch.int32) else level_map_.to(torch.int32)
+    m = m.contiguous()
+    lead, Nk = m.shape[:-1], m.shape[-1]
+    div = max(1, blocksize // compute_tile)
+    out = torch.empty(*lead, Nk + 5, dtype=torch.int32, device=m.device)
+    with torch.cuda.device(m.device):
+        check(lib.psa_list_from_map(_ptr(m), m.element_size(), _ptr(out), m.numel() // Nk, Nk, div, _stream(m)), "psa_list_from_map")
+    return out
+
+
 def k_similarity(k: torch.Tensor, block_n: int, thr2: float, thr4: float, thr8: float) -> torch.Tensor:
     """Per kv-block cap on the pooling level, int32 [B,H,Nk] in {1,2,4,8}."""
     _require_gpu(k)
-    kb = _bf16_view(k)
+    kb = _kernel_view(k, _T16)
     B, H, L, D = kb.shape
     Nk = -(-L // block_n)
     out = torch.empty(B, H, Nk, dtype=torch.int32, device=k.device)
@@ -477,7 +511,7 @@ def sparse_attention_fwd(
     shape has one, False to walk the map itself."""
     _require_gpu(q, k, v, level_map_, q_index)
     in_dtype = q.dtype
-    qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
+    qb, kb, vb = _same_type(_kernel_view(q), _kernel_view(k), _kernel_view(v))
     B, Hq, L, D = qb.shape
     Hkv = kb.shape[1]
     if kb.shape[2] != L or vb.shape != kb.shape or kb.shape[3] != D:
@@ -494,14 +528,18 @@ def sparse_attention_fwd(
         if tuple(level_map_.shape) != (B, Hq, Mq, Nk):
             raise ValueError("level map must be [B, Hq, %d, %d], got %s" % (Mq, Nk, tuple(level_map_.shape)))
         kp, vp = pools if pools is not None else pool_kv(kb, vb, block_n)
-    if out is None or out.dtype != torch.bfloat16:
-        o = torch.empty(B, Hq, L, D, dtype=torch.bfloat16, device=q.device)
+        if kp.dtype != kb.dtype or vp.dtype != kb.dtype:
+            raise ValueError("the pooled buffers must have the element type of k / v (%s)" % kb.dtype)
+    if out is None or out.dtype != qb.dtype:
+        o = torch.empty(B, Hq, L, D, dtype=qb.dtype, device=q.device)
     else:
         o = out
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
     if q_index is not None:
         q_index = _check_index(q_index, L)
-    n_sched = lib.psa_schedule_bytes(B, Hq, Hkv, L, D, block_m, block_n) if (level_map_ is not None and balance and schedule is not False) else 0
+    n_sched = 0
+    if level_map_ is not None and balance and schedule is not False and qb.dtype in _T16:
+        n_sched = lib.psa_schedule_bytes(B, Hq, Hkv, L, D, block_m, block_n)
     if n_sched > 0:
         # the map's tile schedule is built once (one pass over the map) and walked by the kernel
         if not isinstance(schedule, torch.Tensor):
@@ -521,7 +559,7 @@ def sparse_attention_fwd(
                 check(lib.psa_fwd(_t4(qb), *tail), "psa_fwd")
             else:
                 check(lib.psa_fwd_indexed(_t4(qb), _ptr(q_index), *tail), "psa_fwd_indexed")
-    res = o if in_dtype == torch.bfloat16 else o.to(in_dtype)
+    res = o if in_dtype == o.dtype else o.to(in_dtype)
     if return_lse:
         return res, lse, (kp, vp)
     return res
@@ -569,7 +607,7 @@ def psa_layer_fwd(
     (after the re-ordering), and applied to the map; level_cap passes a ready cap instead.  Returns out, or
     (out[, map][, cap]) with return_map / return_cap."""
     _require_gpu(q, k, v)
-    qb, kb, vb = _bf16_view(q), _bf16_view(k), _bf16_view(v)
+    qb, kb, vb = _same_type(_kernel_view(q), _kernel_view(k), _kernel_view(v))
     keep_m, keep_n = block_m // 4, block_n // 4
     sm_scale = qb.shape[-1] ** -0.5 if sm_scale is None else float(sm_scale)
     if token_index is not None:
@@ -583,8 +621,8 @@ def psa_layer_fwd(
         main = torch.cuda.current_stream(qb.device)
         side = _side_stream(qb.device)
         n_pool = lib.psa_pool_elems(kb.shape[0], kb.shape[1], kb.shape[2], kb.shape[3], block_n)
-        kp = torch.empty(n_pool, dtype=torch.bfloat16, device=kb.device)
-        vp = torch.empty(n_pool, dtype=torch.bfloat16, device=kb.device)
+        kp = torch.empty(n_pool, dtype=kb.dtype, device=kb.device)
+        vp = torch.empty(n_pool, dtype=kb.dtype, device=kb.device)
         side.wait_stream(main)
         with torch.cuda.stream(side):
             pool_kv(kb, vb, block_n, out=(kp, vp))
@@ -606,6 +644,58 @@ def psa_layer_fwd(
     if not (return_map or return_cap):
         return out
     return (out,) + ((mp,) if return_map else ()) + ((level_cap,) if return_cap else ())
+
+
+# ----------------------------------------------------------------------------- whole layer as one HIP graph
+_LAYER_GRAPHS: Dict[tuple, tuple] = {}
+_LAYER_GRAPHS_MAX = 16
+
+
+def psa_layer_fwd_graph(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, off_q: torch.Tensor, off_k: torch.Tensor, mask_ratios,
+                        mode: str, block_m: int, block_n: int, tile_n: int, **kwargs):
+    """psa_layer_fwd captured into one HIP graph and replayed: the estimator, the reduction + level map, the tile schedule
+    and the attention kernel on the main branch, the pooling pass on a second branch beside the estimator - kernel nodes
+    only (the library enqueues nothing else: no memset or copy nodes), so the launch gaps and the stream fork / join of
+    the eager sequence disappear.  The graph is tied to the ADDRESSES of q, k, v and the offsets (and to every other
+    argument): a call with tensors at the same addresses replays it on their current contents, any other call captures
+    a new graph (a few are kept).  The returned tensors belong to the graph and are overwritten by its next replay.
+    Same bits as psa_layer_fwd.  Keyword arguments as psa_layer_fwd (tensors among them are part of the key)."""
+    _require_gpu(q, k, v, off_q, off_k)
+
+    def keyof(x):
+        if isinstance(x, torch.Tensor):
+            return ("t", x.data_ptr(), tuple(x.shape), tuple(x.stride()), x.dtype)
+        if isinstance(x, dict):
+            return tuple(sorted((kk, keyof(vv)) for kk, vv in x.items()))
+        if isinstance(x, (list, tuple)):
+            return tuple(keyof(e) for e in x)
+        return x
+
+    key = (keyof((q, k, v, off_q, off_k)), keyof(mask_ratios), mode, block_m, block_n, tile_n, keyof(kwargs),
+           torch.cuda.current_device())
+    ent = _LAYER_GRAPHS.get(key)
+    if ent is None:
+        def run():
+            return psa_layer_fwd(q, k, v, off_q, off_k, mask_ratios, mode, block_m, block_n, tile_n, **kwargs)
+
+        # one eager run first (one-time work such as the check of a token index and the library's function attributes
+        # must not fall into the capture), on a side stream as torch asks for
+        cur = torch.cuda.current_stream(q.device)
+        warm = torch.cuda.Stream(device=q.device)
+        warm.wait_stream(cur)
+        with torch.cuda.stream(warm):
+            run()
+        cur.wait_stream(warm)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            res = run()
+        if len(_LAYER_GRAPHS) >= _LAYER_GRAPHS_MAX:
+            _LAYER_GRAPHS.pop(next(iter(_LAYER_GRAPHS)))
+        # (the key holds addresses only: keep the tensors alive with the graph so that the addresses stay theirs)
+        ent = (graph, res, (q, k, v, off_q, off_k, kwargs))
+        _LAYER_GRAPHS[key] = ent
+    ent[0].replay()
+    return ent[1]
 
 
 # ----------------------------------------------------------------------------- attention backward
@@ -638,7 +728,9 @@ def sparse_attention_bwd(
         level_map_ = level_map_.contiguous()
         if tuple(level_map_.shape) != (B, Hq, Mq, Nk):
             raise ValueError("level map must be [B, Hq, %d, %d], got %s" % (Mq, Nk, tuple(level_map_.shape)))
-        kp, vp = pools if pools is not None and pools[0] is not None else pool_kv(kb, vb, block_n)
+        # (pools of a forward that ran in another element type are of no use to the bf16 kernels here)
+        reuse = pools is not None and pools[0] is not None and pools[0].dtype == torch.bfloat16
+        kp, vp = pools if reuse else pool_kv(kb, vb, block_n)
     lse = lse.to(torch.float32).contiguous()
     if tuple(lse.shape) != (B, Hq, L):
         raise ValueError("lse must be [B, Hq, L]")

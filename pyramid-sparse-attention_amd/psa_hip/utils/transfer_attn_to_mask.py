@@ -1,7 +1,7 @@
 """Scores -> pyramid level mask, and density of a mask.
 
 reference: src/psa_triton/utils/transfer_attn_to_mask.py:6-507 (transfer_attn_to_mask),
-:510-544 (calc_density), :547-622 (calc_density_newtype).
+:510-544 (calc_density), :547-622 (calc_density_newtype), :624-750 (transfer_mask_to_new_type).
 """
 from typing import Dict, Optional, Tuple
 
@@ -43,3 +43,11 @@ def calc_density_newtype(mask: torch.Tensor):
     n_sep = 5
     Nk = mask.shape[-1] - n_sep
     return calc_density(ops.map_from_list(mask, Nk, torch.int8))
+
+
+def transfer_mask_to_new_type(mask: torch.Tensor, blocksize=32, compute_tile=32) -> torch.Tensor:
+    """Dense level mask [B,H,Mq,Nk] (values 0, 1, 2, 4, 8) -> index list [B,H,Mq,Nk+5] int32: the kv-blocks at levels
+    1, 2, 4, 8 and the skipped ones, -1 behind each segment.  Blocks of a level are listed in ascending order (the
+    reference leaves their order to torch.sort); segment lengths are rounded down to the level's alignment
+    ceil(level / (blocksize // compute_tile)), the excess leading the next segment."""
+    return ops.list_from_map(mask, blocksize, compute_tile)

@@ -205,3 +205,46 @@ def test_layer_operator_with_pooling_on_the_second_stream(in_dtype, monkeypatch)
         out, mp = ops.psa_layer_fwd(qd, kd, vd, oq, ok, ratios, "thresholdbound", bm, bn, tn, return_map=True)
         torch.cuda.synchronize()
         assert torch.equal(mp, mp_ref) and torch.equal(out, out_ref) and out.dtype == in_dtype
+
+
+def test_layer_operator_as_one_graph():
+    """psa_layer_fwd_graph: the layer captured into one HIP graph (estimator, reduction + map, schedule, attention; pooling
+    on a second branch) gives the eager layer's bits on every replay, with eager work of the program between replays,
+    follows the CONTENTS of its input tensors, and captures anew for tensors at other addresses."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    B, H, D, bm, bn, tn = 1, 8, 128, 128, 128, 32
+    q, k, v = (t.to(dev()) for t in make_qkv(B, H, H, (8, 16, 32), D, seed=11))  # 4096 tokens: K is 8 MiB
+    oq, ok = sample_offsets(B, H, bm, 32, 12).to(dev()), sample_offsets(B, H, bn, 32, 13).to(dev())
+    ratios = {1: (0.0, 0.3), 2: (0.3, 0.4), 4: (0.4, 0.5), 8: (0.5, 0.6), 0: (0.6, 1.0)}
+    for side_min in (0, 1 << 40):  # with and without the second branch for the pooling pass
+        ops._SIDE_STREAM_MIN_BYTES, saved = side_min, ops._SIDE_STREAM_MIN_BYTES
+        try:
+            ops._LAYER_GRAPHS.clear()
+            ref, ref_map = ops.psa_layer_fwd(q, k, v, oq, ok, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+            ref, ref_map = ref.clone(), ref_map.clone()
+            for rep in range(3):
+                junk = torch.randn(1 << 20, device=dev()).sum()
+                torch.cuda.synchronize()
+                out, mp = ops.psa_layer_fwd_graph(q, k, v, oq, ok, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+                torch.cuda.synchronize()
+                assert torch.equal(out, ref) and torch.equal(mp, ref_map), (side_min, rep)
+                assert torch.isfinite(junk)
+            assert len(ops._LAYER_GRAPHS) == 1
+            # new contents at the same addresses: the replay computes the new layer
+            q2 = torch.roll(q, 17, dims=2).contiguous()
+            ref2 = ops.psa_layer_fwd(q2, k, v, oq, ok, ratios, "thresholdbound", bm, bn, tn).clone()
+            q_saved = q.clone()
+            q.copy_(q2)
+            out2, _ = ops.psa_layer_fwd_graph(q, k, v, oq, ok, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+            torch.cuda.synchronize()
+            assert torch.equal(out2, ref2) and len(ops._LAYER_GRAPHS) == 1
+            q.copy_(q_saved)
+            # other tensors: another graph
+            out3, _ = ops.psa_layer_fwd_graph(q2, k, v, oq, ok, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+            torch.cuda.synchronize()
+            assert torch.equal(out3, ref2) and len(ops._LAYER_GRAPHS) == 2
+        finally:
+            ops._SIDE_STREAM_MIN_BYTES = saved
+            ops._LAYER_GRAPHS.clear()

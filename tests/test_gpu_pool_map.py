@@ -131,3 +131,22 @@ def test_map_from_list_and_min_cap():
     assert np.array_equal(m.cpu().numpy(), np.minimum(dense, cap.cpu().numpy()[:, :, None, :]))
     dc = ops.density(m, causal=False)
     assert abs(float(dc[-1]) - O.density(m.cpu().numpy())) < 1e-6
+
+
+@pytest.mark.parametrize("blocksize,tile", [(32, 32), (128, 32), (64, 32), (128, 64)])
+def test_dense_map_to_index_list_bit_exact(blocksize, tile):
+    from psa_hip import ops
+    from psa_hip.utils import transfer_mask_to_new_type
+
+    rng = np.random.default_rng(blocksize + tile)
+    m = rng.choice([0, 1, 2, 4, 8], size=(2, 3, 9, 300), p=(0.4, 0.2, 0.15, 0.15, 0.1)).astype(np.int32)
+    m[0, 0, 0] = 0
+    m[0, 0, 1] = 1
+    m[0, 0, 2] = 8
+    for dt in (torch.int32, torch.int8):
+        got = transfer_mask_to_new_type(torch.from_numpy(m).to(dt).to(dev()), blocksize, tile)
+        assert got.dtype == torch.int32 and tuple(got.shape) == (2, 3, 9, 305)
+        assert np.array_equal(got.cpu().numpy(), O.dense_to_list(m, blocksize, tile))
+    # and back through the list import
+    back = ops.map_from_list(got, 300, torch.int32).cpu().numpy()
+    assert np.array_equal(back, O.list_to_dense(O.dense_to_list(m, blocksize, tile), 300))

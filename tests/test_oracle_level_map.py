@@ -132,3 +132,32 @@ def test_errors():
         O.level_map(np.ones((1, 1, 1, 4), np.float32), None)
     with pytest.raises(ValueError):
         O.level_map(np.ones((1, 1, 1, 4), np.float32), WAN14, mode="nope")
+
+
+def test_dense_to_list_hand_worked_and_round_trip():
+    """dense map -> index list (transfer_mask_to_new_type): a hand-worked row with the alignment rule, and the round trip
+    through the list-walking rule of the attention kernel."""
+    #            j: 0  1  2  3  4  5  6  7  8  9
+    row = np.array([1, 0, 2, 8, 1, 2, 4, 2, 1, 8], np.int32)
+    # blocksize == compute_tile: level l segments hold multiples of l.  Sorted by level: 1:[0,4,8] 2:[2,5,7] 4:[6] 8:[3,9] 0:[1]
+    #   level 1: 3 blocks, multiple of 1 -> [0,4,8]
+    #   level 2: 3 blocks -> 2 stay [2,5], block 7 leads the next segment
+    #   level 4: [7,6] is 2 blocks -> 0 stay, both move on
+    #   level 8: [7,6,3,9] is 4 blocks -> 0 stay, all move to the skipped segment
+    lst = O.dense_to_list(row.reshape(1, -1), 32, 32).reshape(-1).tolist()
+    assert lst == [0, 4, 8, -1, 2, 5, -1, -1, -1, 7, 6, 3, 9, 1, -1]
+    # blocksize 128, compute tile 32: every alignment is ceil(level / 4) -> 1, 1, 1, 2
+    lst = O.dense_to_list(row.reshape(1, -1), 128, 32).reshape(-1).tolist()
+    assert lst == [0, 4, 8, -1, 2, 5, 7, -1, 6, -1, 3, 9, -1, 1, -1]
+    rng = np.random.default_rng(0)
+    m = rng.choice([0, 1, 2, 4, 8], size=(2, 3, 7, 40)).astype(np.int32)
+    lst = O.dense_to_list(m, 128, 32)
+    assert lst.shape == (2, 3, 7, 45) and (lst == -1).sum(-1).min() == 5 and (lst == -1).sum(-1).max() == 5
+    back = O.list_to_dense(lst, 40)
+    # without excess (alignment 1 for levels 1-4, level-8 segments rounded down to even) the walk reads the map back,
+    # except for a level-8 block that moved into the skipped segment
+    moved = (back != m)
+    assert np.all(m[moved] == 8) and np.all(back[moved] == 0) and moved.sum(-1).max() <= 1
+    # every block is listed exactly once
+    body = np.sort(np.where(lst == -1, 10 ** 6, lst), -1)[..., :40]
+    assert np.array_equal(body, np.broadcast_to(np.arange(40), body.shape))
