@@ -21,17 +21,17 @@ sys.path.insert(0, PKG)
 
 METRIC = "PSA attn ms/layer + effective TFLOPS (% bf16 MFMA peak) at Wan2.1-1.3B shape, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
     # BASELINE.json configs[1]: Wan2.1-1.3B 480p self-attention layer
     "c2": dict(name="wan2.1-1.3b-480p B1 H12 N32760 D128 bf16 blk128 thresholdbound ~90% sparsity",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.90),
-    # BASELINE.json configs[0] (small; the configuration names fp32 - the kernels compute on bf16 operands with fp32
-    # accumulation, fp32 inputs are rounded to bf16 on entry, and the JSON line says so in `dtype`)
-    "c1": dict(name="small B1 H2 N4096 D64 blk64 thresholdbound ~80% sparsity",
-               B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80,
-               dtype="bf16 (the configuration names fp32: inputs are rounded to bf16 on entry)"),
+    # BASELINE.json configs[0] (small, fp32 tensors: every stage computes in fp32 - the fp32 kernels run on the vector
+    # units, so the peak its roofline line is priced against is the fp32 one)
+    "c1": dict(name="small B1 H2 N4096 D64 fp32 blk64 thresholdbound ~80% sparsity",
+               B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80, dtype="fp32"),
 }
 WORKLOADS.update({
     # BASELINE.json configs[2]: CogVideoX-5B joint text + video attention (text blocks last, always level 1)
@@ -274,7 +274,9 @@ def main():
         return
     B, H, D, bm, bn, tn = w["B"], w["H"], w["D"], w["bm"], w["bn"], w["tn"]
     text = w.get("text", 0)
-    q, k, v = make_qkv(B, H, H, w["grid"], D, seed=args.seed, device=dev, text_tokens=text)
+    tdtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[w.get("dtype", "bf16")]
+    peak = PEAK_FP32_TFLOPS if tdtype == torch.float32 else PEAK_BF16_TFLOPS
+    q, k, v = make_qkv(B, H, H, w["grid"], D, seed=args.seed, device=dev, text_tokens=text, dtype=tdtype)
     L = q.shape[2]
     Mq, Nk = -(-L // bm), -(-L // bn)
     km, kn = bm // 4, bn // 4
@@ -403,16 +405,17 @@ def main():
             preset = {"module_layer": round(t_mod, 4), "k_similarity": round(t_ks, 4),
                       "what": "PyramidSparseAttention.forward, Gilbert re-ordering through the token index + similarity cap"}
 
-    pool_bytes = 2.0 * B * H * (Nk * bn) * D * 2 * (1 + 7 / 8)
+    pool_bytes = 2.0 * B * H * (Nk * bn) * D * q.element_size() * (1 + 7 / 8)
     est_flops = 2.0 * (Mq * km) * (Nk * kn) * D * B * H
 
     roofline = {
-        "kernel": "psa_fwd_pp_kernel" if (D == 128 and bm == 128) else "psa_fwd_lds_kernel",
-        "bound": "mfma",
+        "kernel": ("psa_fwd_f32_kernel" if tdtype == torch.float32 else
+                   "psa_fwd_pp_kernel" if (D == 128 and bm == 128) else "psa_fwd_lds_kernel"),
+        "bound": "mfma",  # (the fp32 kernel computes on the vector units; its peak is the fp32 figure)
         "achieved": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12, 2),
-        "peak": PEAK_BF16_TFLOPS,
+        "peak": peak,
         "unit": "TFLOP/s",
-        "frac": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+        "frac": round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / peak, 4),
         # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command (scaled by the
         # readings of --copy-calib's 1 GiB kernel); measured for the default workload only
         "traffic": fwd_traffic_bytes(args.workload),
@@ -465,7 +468,8 @@ def main():
             "host_cpus": ncores,
             "kind": "port",
             "repetitions": 3 if (len(heads) == H and len(qblocks) == Mq) else 1,
-            # the GPU layer's output against the oracle's on the rows the oracle computed (bf16 tolerance: 2e-2 / 2e-3)
+            # the GPU layer's output against the oracle's (run on the same tensors, in fp32) on the rows the oracle computed
+            # (tolerance of the 16-bit types: 2e-2 / 2e-3)
             "max_abs": round(cpu_max_abs, 5), "mean_abs": round(cpu_mean_abs, 6),
             "sample": ("the whole layer in fp32: all %d heads, all %d q-blocks (estimate + level map + attention), minimum of 3" % (H, Mq))
             if len(heads) == H and len(qblocks) == Mq else

@@ -109,6 +109,9 @@ def _check_index(index: torch.Tensor, L: int) -> torch.Tensor:
     if index.dtype != torch.int32 or index.dim() != 1 or index.numel() != L:
         raise ValueError("index must be a 1-D int32 tensor with one entry per token (%d)" % L)
     index = index.contiguous()
+    if index.is_inference():  # no version counter to key a cached verdict on: checked on every call
+        validate_token_index(index, L)
+        return index
     key = (index.data_ptr(), index._version, L, index.device.index if index.device.index is not None else -1)
     if key not in _VALID_INDEX:
         validate_token_index(index, L)

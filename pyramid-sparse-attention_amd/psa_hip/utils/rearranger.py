@@ -39,11 +39,14 @@ class GilbertRearranger:
         key = (str(device), forward, "combined")
         if key not in self._cache:
             t, n = self.text_length, self.total_elements
-            if forward:
-                idx = torch.cat((self.original_order2gilbert_order_cpu + t, torch.arange(t)))
-            else:
-                idx = torch.cat((torch.arange(t) + n, self.gilbert_order2original_order_cpu))
-            self._cache[key] = idx.to(torch.int32).to(device)
+            # (built as an ordinary tensor also when first asked for under torch.inference_mode: the operators cache their
+            # validity check of an index on its version counter, which inference tensors do not have)
+            with torch.inference_mode(False):
+                if forward:
+                    idx = torch.cat((self.original_order2gilbert_order_cpu + t, torch.arange(t)))
+                else:
+                    idx = torch.cat((torch.arange(t) + n, self.gilbert_order2original_order_cpu))
+                self._cache[key] = idx.to(torch.int32).to(device)
         return self._cache[key]
 
     def token_index(self, device) -> torch.Tensor:

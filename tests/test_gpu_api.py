@@ -248,3 +248,28 @@ def test_layer_operator_as_one_graph():
         finally:
             ops._SIDE_STREAM_MIN_BYTES = saved
             ops._LAYER_GRAPHS.clear()
+
+
+def test_token_index_made_under_inference_mode():
+    """An index tensor created under torch.inference_mode has no version counter: its contents are checked on every
+    call instead of once, and the operators take it like any other."""
+    from psa_hip import ops
+    from psa_hip.utils.rearranger import GilbertRearranger
+
+    L = 4 * 6 * 8
+    k, v = rnd(1, 2, L, 128, seed=1).to(dev()), rnd(1, 2, L, 128, seed=2).to(dev())
+    with torch.inference_mode():
+        rr = GilbertRearranger(8, 6, 4, 0)
+        idx = rr.token_index(dev())
+        raw = idx.clone()  # an inference tensor
+        assert raw.is_inference() and not idx.is_inference()
+        a = ops.pool_kv_indexed(k, v, idx, 32)
+        b = ops.pool_kv_indexed(k, v, raw, 32)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    bad = raw.clone()
+    with torch.inference_mode():
+        worse = bad.clone()
+        worse[3] = worse[4]
+        with pytest.raises(ValueError):
+            ops.pool_kv_indexed(k, v, worse, 32)
