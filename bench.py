@@ -68,7 +68,7 @@ def scaled_ratios(tau):
     return {lv: (lo * tau if lv else 0.8 * tau, hi * tau if lv else 1.0) for lv, (lo, hi) in WAN13.items()}
 
 
-def time_gpu(fn, iters, warm=3):
+def time_gpu(fn, iters, warm=20):
     import torch
 
     for _ in range(warm):
@@ -82,6 +82,42 @@ def time_gpu(fn, iters, warm=3):
     torch.cuda.synchronize()
     ts = sorted(a.elapsed_time(b) for a, b in evs)
     return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def sclk_under_load(fn, ms_per_call):
+    """Shader clock (MHz) that rocm-smi reports while fn runs back to back for about 1.5 s: the clock the launch's cycles
+    are counted in (the published peak is quoted at the 2400 MHz maximum).  None when rocm-smi gives no reading."""
+    import re
+    import subprocess
+    import threading
+
+    import torch
+
+    reads, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+                m = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", out)
+                if m:
+                    reads.append(int(m.group(1)))
+            except Exception:
+                return
+            stop.wait(0.1)
+
+    th = threading.Thread(target=poll, daemon=True)
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    th.start()
+    for _ in range(max(10, int(1500.0 / max(ms_per_call, 1e-3)))):
+        fn()
+    torch.cuda.synchronize()
+    stop.set()
+    th.join(timeout=30)
+    reads = sorted(reads[1:] or reads)  # (the first reading may predate the load)
+    return reads[len(reads) // 2] if reads else None
 
 
 def copy_calib(torch, dev):
@@ -352,7 +388,9 @@ def main():
     if ops.lib.psa_schedule_bytes(B, H, H, L, D, bm, bn) > 0:
         sched = ops.build_schedule(mp, H, L, D, bm, bn)
         t_sched, _ = time_gpu(lambda: ops.build_schedule(mp, H, L, D, bm, bn, out=sched), it)
-    t_fwd_med, t_fwd_avg = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf, schedule=sched), it)
+    fwd_call = lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf, schedule=sched)
+    t_fwd_med, t_fwd_avg = time_gpu(fwd_call, it)
+    sclk = None if args.no_extras else sclk_under_load(fwd_call, t_fwd_avg)
     t_dense = t_sdpa = None
     if not args.no_dense:
         t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
@@ -421,6 +459,10 @@ def main():
         "traffic": fwd_traffic_bytes(args.workload),
         "flops_per_launch": exec_flops,
         "avg_launch_ms": round(t_fwd_avg, 4),
+        # context, not the fraction that counts: the shader clock under this kernel (the board's power limit holds it under
+        # the 2400 MHz the peak is quoted at) and the fraction of the peak scaled to that clock
+        "sclk_mhz_under_load": sclk,
+        "frac_at_that_clock": None if not sclk else round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / (peak * sclk / 2400.0), 4),
         "launch_includes": ("the forward kernel alone (it walks the map's prebuilt tile schedule: stages_ms.schedule)" if sched is not None
                             else "the forward kernel and its two row-ordering launches"),
     }

@@ -9,11 +9,11 @@
 // Four kernels:
 //   psa_bwd_delta_kernel   HBM-bound: delta and lse in log2 units (rows without keys get +inf so p = 0)
 //   psa_bwd_dq_lds_kernel  MFMA-bound row walk: the forward's tile schedule; per tile S^T = K Q^T,
-//                          dP^T = V dO^T, dQ^T += K^T dS^T on bf16 MFMA, operands pooled K/V read directly
+//                          dP^T = V dO^T, dQ^T += K^T dS^T on bf16 / fp16 MFMA, operands pooled K/V read directly
 //   psa_bwd_dkdv_lds_kernel MFMA-bound column walk: one workgroup per (kv head, kv-block, level slot) keeps its
 //                          <= 64 pooled keys in registers and streams the q-blocks that retain this block at
 //                          this level; dK_l, dV_l go to an fp32 workspace (every row written exactly once)
-//   psa_bwd_unpool_kernel  HBM-bound: sums the levels, spreads pooled gradients, folds the pad tail, -> bf16
+//   psa_bwd_unpool_kernel  HBM-bound: sums the levels, spreads pooled gradients, folds the pad tail, -> the tensors' type
 #include <type_traits>
 
 #include "psa_tiles.h"
@@ -44,7 +44,7 @@ struct BwdParams {
 // ------------------------------------------------------------------------------------------------------
 // delta and log2-domain lse
 // ------------------------------------------------------------------------------------------------------
-template <int D>
+template <int D, class ET>
 __global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
   constexpr int LPR = D / 8;  // lanes per row
   const int bh = blockIdx.y, b = bh / p.Hq, h = bh % p.Hq;
@@ -56,8 +56,8 @@ __global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
     const u32x4 dw = *(const u32x4*)(p.dout + b * p.do_sb + h * p.do_sh + row * p.do_sl + c * 8);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      acc += bf16_bits_to_f32(ow[j] & 0xffffu) * bf16_bits_to_f32(dw[j] & 0xffffu);
-      acc += __builtin_bit_cast(float, ow[j] & 0xffff0000u) * __builtin_bit_cast(float, dw[j] & 0xffff0000u);
+      acc += ET::from_bits(ow[j] & 0xffffu) * ET::from_bits(dw[j] & 0xffffu);
+      acc += ET::from_bits(ow[j] >> 16) * ET::from_bits(dw[j] >> 16);
     }
   }
 #pragma unroll
@@ -75,9 +75,10 @@ __global__ __launch_bounds__(256) void psa_bwd_delta_kernel(BwdParams p) {
 // into double-buffered LDS tiles (layout: psa_tiles.h), one barrier per tile; S^T = K Q^T and dP^T = V dO^T
 // read them row-wise (128-bit reads), dQ^T += K^T dS^T reads the K tile through the transposing LDS load.
 // ------------------------------------------------------------------------------------------------------
-template <int D, int NW>
+template <int D, int NW, class ET>
 __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p, int chunk, const int32_t* order) {
   using G = LtGeom<D>;
+  using x8 = typename ET::x8;
   constexpr int LT_TILE = G::TILE;
   constexpr int NT = NW * 64, BM = NW * 32, CH = D / 8, KK = D / 16, DB = D / 32;
   constexpr int G16 = 4 / NW;
@@ -111,14 +112,14 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p,
   // Q and dO fragments of this wave's 32 rows (B operands), per-row delta and lse
   const int q_idx = I * BM + wave * 32 + l32;
   const int qr = q_idx < L ? q_idx : L - 1;
-  bf16x8 qf[KK], dof[KK];
+  x8 qf[KK], dof[KK];
   {
     const bf16_t* qp = p.q + b * p.q_sb + h * p.q_sh + (int64_t)qr * p.q_sl + hh * 8;
     const bf16_t* dp_ = p.dout + b * p.do_sb + h * p.do_sh + (int64_t)qr * p.do_sl + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      qf[kk] = *(const bf16x8*)(qp + kk * 16);
-      dof[kk] = *(const bf16x8*)(dp_ + kk * 16);
+      qf[kk] = *(const x8*)(qp + kk * 16);
+      dof[kk] = *(const x8*)(dp_ + kk * 16);
     }
   }
   const float delta = q_idx < L ? p.delta[(int64_t)bh * L + q_idx] : 0.f;
@@ -170,10 +171,10 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p,
     for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        const bf16x8 ka = *(PSA_LDS(const bf16x8))(Ks + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
-        s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s[c], 0, 0, 0);
-        const bf16x8 va = *(PSA_LDS(const bf16x8))(Vs + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
-        dp[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[kk], dp[c], 0, 0, 0);
+        const x8 ka = *(PSA_LDS(const x8))(Ks + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
+        s[c] = ET::mfma(ka, qf[kk], s[c]);
+        const x8 va = *(PSA_LDS(const x8))(Vs + r_off[kk & 1] + (kk >> 1) * 64 + c * G::HALF);
+        dp[c] = ET::mfma(va, dof[kk], dp[c]);
       }
     }
     if (d & 4) {
@@ -209,20 +210,20 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p,
       for (int i = 0; i < 16; i += 2) {
         const float p0 = fast_exp2(__builtin_fmaf(s[c][i], scale_log2, nb));
         const float p1 = fast_exp2(__builtin_fmaf(s[c][i + 1], scale_log2, nb));
-        pk[c][i >> 1] = pack_bf16x2(p0 * (dp[c][i] - delta), p1 * (dp[c][i + 1] - delta));
+        pk[c][i >> 1] = ET::pack2(p0 * (dp[c][i] - delta), p1 * (dp[c][i + 1] - delta));
       }
     // dQ^T += K^T dS^T
 #pragma unroll
     for (int cg = 0; cg < 4; ++cg) {
       const int c = cg >> 1, g = cg & 1;
       u32x4 bw = {pk[c][g * 4 + 0], pk[c][g * 4 + 1], pk[c][g * 4 + 2], pk[c][g * 4 + 3]};
-      const bf16x8 bfrag = __builtin_bit_cast(bf16x8, bw);
+      const x8 bfrag = __builtin_bit_cast(x8, bw);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[0] + db * 64 + cg * G::GROUP)));
-        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Ks + t_off[1] + db * 64 + cg * G::GROUP)));
+        const u32x2 lo = ET::read_tr(Ks + t_off[0] + db * 64 + cg * G::GROUP);
+        const u32x2 hi = ET::read_tr(Ks + t_off[1] + db * 64 + cg * G::GROUP);
         u32x4 aw = {lo[0], lo[1], hi[0], hi[1]};
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aw), bfrag, acc[db], 0, 0, 0);
+        acc[db] = ET::mfma(__builtin_bit_cast(x8, aw), bfrag, acc[db]);
       }
     }
   };
@@ -259,8 +260,8 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_bwd_dq_lds_kernel(BwdParams p,
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x2 w;
-      w[0] = pack_bf16x2(acc[db][g * 4 + 0] * scale, acc[db][g * 4 + 1] * scale);
-      w[1] = pack_bf16x2(acc[db][g * 4 + 2] * scale, acc[db][g * 4 + 3] * scale);
+      w[0] = ET::pack2(acc[db][g * 4 + 0] * scale, acc[db][g * 4 + 1] * scale);
+      w[1] = ET::pack2(acc[db][g * 4 + 2] * scale, acc[db][g * 4 + 3] * scale);
       *(u32x2*)(Os + (wave * 32 + l32) * OST + (db * 32 + g * 8 + hh * 4) * 2) = w;
     }
   __syncthreads();
@@ -331,10 +332,11 @@ constexpr int B_ISTR = LT_ISTR;  // bytes between the blocks of a tile
 // One instantiation per kind of slot (WIDE: the 128-key level-0 slot; else the slots slot_lo .. slot_lo + slot_cnt - 1 of
 // every kv-block); workgroup id = ((b * Hkv + kv head) * Nk + kv-block) * slot_cnt + (slot - slot_lo), optionally
 // re-ordered.
-template <int D, bool WIDE, bool CAUSAL>
+template <int D, bool WIDE, bool CAUSAL, class ET>
 __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, int slot_lo, int slot_cnt, int n_wg, int chunk,
                                                                  const int32_t* order) {
   using G = LtGeom<D>;
+  using x8 = typename ET::x8;
   constexpr int KK = D / 16, DB = D / 32, RPL = G::RPL;
   constexpr int B_TILE = G::TILE;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -398,7 +400,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
 
   // ---- this wave's 32 keys: K and V fragments (B operands) --------------------------------------------
   const int key_local = kh * 32 + l32;
-  bf16x8 kf[KK], vf[KK];
+  x8 kf[KK], vf[KK];
   {
     int64_t row = key_row0 + (key_local < key_valid ? key_local : 0);
     if (key_valid == 0) row = 0;
@@ -415,8 +417,8 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      kf[kk] = *(const bf16x8*)(kp_ + kk * 16 + hh * 8);
-      vf[kk] = *(const bf16x8*)(vp_ + kk * 16 + hh * 8);
+      kf[kk] = *(const x8*)(kp_ + kk * 16 + hh * 8);
+      vf[kk] = *(const x8*)(vp_ + kk * 16 + hh * 8);
     }
   }
   const int key_up = (int)(((key_row0 + key_local + 1) << lv) - 1);  // last token the pooled key covers (< npad)
@@ -528,10 +530,10 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
     }
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      const bf16x8 qa = *(PSA_LDS(const bf16x8))(Qs + r_off[kk & 1] + (kk >> 1) * 64);
-      const bf16x8 oa = *(PSA_LDS(const bf16x8))(Os + r_off[kk & 1] + (kk >> 1) * 64);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
-      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[kk], dp, 0, 0, 0);
+      const x8 qa = *(PSA_LDS(const x8))(Qs + r_off[kk & 1] + (kk >> 1) * 64);
+      const x8 oa = *(PSA_LDS(const x8))(Os + r_off[kk & 1] + (kk >> 1) * 64);
+      s = ET::mfma(qa, kf[kk], s);
+      dp = ET::mfma(oa, vf[kk], dp);
     }
     uint32_t pk[8], dsk[8];
     // p = exp2(scale * s + bias - lse), dS = p (dP - delta).  Lanes whose key does not exist (the ragged end of the
@@ -554,28 +556,28 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
         pv[e2] = pe;
         dsv[e2] = pe * (dp[g * 4 + e2] - d4[e2]);
       }
-      pk[g * 2] = pack_bf16x2(pv[0], pv[1]);
-      pk[g * 2 + 1] = pack_bf16x2(pv[2], pv[3]);
-      dsk[g * 2] = pack_bf16x2(dsv[0], dsv[1]);
-      dsk[g * 2 + 1] = pack_bf16x2(dsv[2], dsv[3]);
+      pk[g * 2] = ET::pack2(pv[0], pv[1]);
+      pk[g * 2 + 1] = ET::pack2(pv[2], pv[3]);
+      dsk[g * 2] = ET::pack2(dsv[0], dsv[1]);
+      dsk[g * 2 + 1] = ET::pack2(dsv[2], dsv[3]);
     }
     // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over this wave's 32 query rows, 16 at a time)
 #pragma unroll
     for (int g = 0; g < 2; ++g) {
       u32x4 pw = {pk[g * 4 + 0], pk[g * 4 + 1], pk[g * 4 + 2], pk[g * 4 + 3]};
       u32x4 sw = {dsk[g * 4 + 0], dsk[g * 4 + 1], dsk[g * 4 + 2], dsk[g * 4 + 3]};
-      const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pw), sfrag = __builtin_bit_cast(bf16x8, sw);
+      const x8 pfrag = __builtin_bit_cast(x8, pw), sfrag = __builtin_bit_cast(x8, sw);
       const int grp = g * G::GROUP;  // (Qs, Os already point at this pass's query half = two 16-row groups)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const u32x2 olo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[0] + db * 64 + grp)));
-        const u32x2 ohi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Os + t_off[1] + db * 64 + grp)));
+        const u32x2 olo = ET::read_tr(Os + t_off[0] + db * 64 + grp);
+        const u32x2 ohi = ET::read_tr(Os + t_off[1] + db * 64 + grp);
         u32x4 oa = {olo[0], olo[1], ohi[0], ohi[1]};
-        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, oa), pfrag, dv[db], 0, 0, 0);
-        const u32x2 qlo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Qs + t_off[0] + db * 64 + grp)));
-        const u32x2 qhi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((PSA_LDS(bf16x4))(Qs + t_off[1] + db * 64 + grp)));
+        dv[db] = ET::mfma(__builtin_bit_cast(x8, oa), pfrag, dv[db]);
+        const u32x2 qlo = ET::read_tr(Qs + t_off[0] + db * 64 + grp);
+        const u32x2 qhi = ET::read_tr(Qs + t_off[1] + db * 64 + grp);
         u32x4 qa2 = {qlo[0], qlo[1], qhi[0], qhi[1]};
-        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qa2), sfrag, dk[db], 0, 0, 0);
+        dk[db] = ET::mfma(__builtin_bit_cast(x8, qa2), sfrag, dk[db]);
       }
     }
     if (WIDE) __builtin_amdgcn_sched_barrier(0);  // the second pass starts after the first: its operands do not fit beside it
@@ -608,7 +610,7 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
 
   // ---- 128-key level-0 slot: this workgroup owns 128 tokens of dK / dV outright.  The pooled levels' launch has
   // finished, so the tokens' shares of the pooled gradients (1/l of pooled row n >> level; for the last real token
-  // also those of the replicate-pad tokens behind it) are added here and dK, dV leave as bf16: no fp32 level-0
+  // also those of the replicate-pad tokens behind it) are added here and dK, dV leave in the tensors' 16-bit type: no fp32 level-0
   // buffer, no separate pass.  Same sums in the same order as psa_bwd_unpool_kernel.
   if constexpr (WIDE) {
     const int64_t n = key_row0 + key_local;
@@ -666,10 +668,10 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
             }
           }
           u32x2 ok_, ov_;
-          ok_[0] = pack_bf16x2(gk[0], gk[1]);
-          ok_[1] = pack_bf16x2(gk[2], gk[3]);
-          ov_[0] = pack_bf16x2(gv[0], gv[1]);
-          ov_[1] = pack_bf16x2(gv[2], gv[3]);
+          ok_[0] = ET::pack2(gk[0], gk[1]);
+          ok_[1] = ET::pack2(gk[2], gk[3]);
+          ov_[0] = ET::pack2(gv[0], gv[1]);
+          ov_[1] = ET::pack2(gv[2], gv[3]);
           *(u32x2*)(dkp + col) = ok_;
           *(u32x2*)(dvp + col) = ov_;
         }
@@ -714,8 +716,9 @@ __global__ __launch_bounds__(256, 2) void psa_bwd_dkdv_lds_kernel(BwdParams p, i
 }
 
 // ------------------------------------------------------------------------------------------------------
-// un-pool: levels -> dK, dV (bf16)
+// un-pool: levels -> dK, dV (the tensors' 16-bit type)
 // ------------------------------------------------------------------------------------------------------
+template <class ET>
 __global__ __launch_bounds__(256) void psa_bwd_unpool_kernel(BwdParams p, int D) {
   const int which = blockIdx.z;  // 0: dK, 1: dV
   const int bhk = blockIdx.y, b = bhk / p.Hkv, hk = bhk % p.Hkv;
@@ -756,8 +759,8 @@ __global__ __launch_bounds__(256) void psa_bwd_unpool_kernel(BwdParams p, int D)
   }
   bf16_t* dst = which == 0 ? p.dk + b * p.dk_sb + hk * p.dk_sh + n * p.dk_sl : p.dv + b * p.dv_sb + hk * p.dv_sh + n * p.dv_sl;
   u32x2 o;
-  o[0] = pack_bf16x2(g[0], g[1]);
-  o[1] = pack_bf16x2(g[2], g[3]);
+  o[0] = ET::pack2(g[0], g[1]);
+  o[1] = ET::pack2(g[2], g[3]);
   *(u32x2*)(dst + c * 4) = o;
 }
 
@@ -799,6 +802,10 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   const int Mq = (L + block_m - 1) / block_m, Nk = (L + block_n - 1) / block_n;
   PSA_REQUIRE(Nk <= 65535 && Mq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: more than 65535 blocks");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_bwd: B*Hq too large");
+  for (int i = 1; i < 8; ++i)
+    PSA_REQUIRE(ts[i]->dtype == q.dtype, PSA_ERR_ARG, "psa_bwd: q, k, v, out, dout, dq, dk, dv must share one element type");
+  PSA_REQUIRE(q.dtype == PSA_DTYPE_BF16 || q.dtype == PSA_DTYPE_F16, PSA_ERR_UNSUPPORTED,
+              "psa_bwd: element type must be bf16 or fp16 (the pooled buffers in the same type)");
   BwdParams p;
   p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr; p.v = (const bf16_t*)v.ptr;
   p.o = (const bf16_t*)out.ptr; p.dout = (const bf16_t*)dout.ptr;
@@ -827,12 +834,14 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   p.lse2 = p.delta + (int64_t)B * Hq * L;
   hipStream_t st = (hipStream_t)stream;
 
+  auto run = [&](auto et) -> int {
+  using ET = decltype(et);
   // 1. delta, lse2
   {
     const int rows_per_wg = 256 / (D / 8);
     dim3 grid((unsigned)((L + rows_per_wg - 1) / rows_per_wg), (unsigned)(B * Hq));
-    if (D == 128) hipLaunchKernelGGL(psa_bwd_delta_kernel<128>, grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(psa_bwd_delta_kernel<64>, grid, dim3(256), 0, st, p);
+    if (D == 128) hipLaunchKernelGGL((psa_bwd_delta_kernel<128, ET>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((psa_bwd_delta_kernel<64, ET>), grid, dim3(256), 0, st, p);
     const int rc = psa_check_launch("psa_bwd (delta)");
     if (rc != PSA_OK) return rc;
   }
@@ -866,10 +875,10 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
       return PSA_OK;
     };
     int rc;
-    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 4>, (size_t)4 * LtGeom<128>::TILE, 4);
-    else if (D == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 2>, (size_t)4 * LtGeom<128>::TILE, 2);
-    else if (block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<64, 4>, (size_t)4 * LtGeom<64>::TILE, 4);
-    else rc = launch(psa_bwd_dq_lds_kernel<64, 2>, (size_t)4 * LtGeom<64>::TILE, 2);
+    if (D == 128 && block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 4, ET>, (size_t)4 * LtGeom<128>::TILE, 4);
+    else if (D == 128) rc = launch(psa_bwd_dq_lds_kernel<128, 2, ET>, (size_t)4 * LtGeom<128>::TILE, 2);
+    else if (block_m == 128) rc = launch(psa_bwd_dq_lds_kernel<64, 4, ET>, (size_t)4 * LtGeom<64>::TILE, 4);
+    else rc = launch(psa_bwd_dq_lds_kernel<64, 2, ET>, (size_t)4 * LtGeom<64>::TILE, 2);
     PSA_REQUIRE(rc == PSA_OK, rc, "psa_bwd: sequence too long for the on-chip schedule (LDS)");
     rc = psa_check_launch("psa_bwd (dQ)");
     if (rc != PSA_OK) return rc;
@@ -915,20 +924,20 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
     const int lo = wide0 ? 1 : 0;
     int rl;
     if (causal)
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, true, ET>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, true, ET>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
     else
-      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
-                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
+      rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, false, false, ET>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest)
+                    : launch(psa_bwd_dkdv_lds_kernel<64, false, false, ET>, n_rest, chunk_r, groups_r, lo, DKDV_SLOTS - lo, order_rest);
     PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
     if (int e = psa_check_launch("psa_bwd (dK/dV)")) return e;
     if (wide0) {
       if (causal)
-        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
-                      : launch(psa_bwd_dkdv_lds_kernel<64, true, true>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, true, ET>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, true, ET>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
       else
-        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
-                      : launch(psa_bwd_dkdv_lds_kernel<64, true, false>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
+        rl = D == 128 ? launch(psa_bwd_dkdv_lds_kernel<128, true, false, ET>, n_wide, chunk_w, groups_w, 0, 1, order_wide)
+                      : launch(psa_bwd_dkdv_lds_kernel<64, true, false, ET>, n_wide, chunk_w, groups_w, 0, 1, order_wide);
       PSA_REQUIRE(rl == PSA_OK, rl, "psa_bwd: cannot reserve %zu bytes of LDS", shmem);
       return psa_check_launch("psa_bwd (dK/dV, 128-key slots)");
     }
@@ -937,7 +946,11 @@ extern "C" int psa_bwd(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* 
   {
     const int64_t units = (int64_t)L * (D / 4);
     dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * Hkv), 2);
-    hipLaunchKernelGGL(psa_bwd_unpool_kernel, grid, dim3(256), 0, st, p, D);
+    hipLaunchKernelGGL(psa_bwd_unpool_kernel<ET>, grid, dim3(256), 0, st, p, D);
   }
   return psa_check_launch("psa_bwd (un-pool)");
+  };
+  int rc = PSA_ERR_ARG;
+  psa_dispatch16(q.dtype, [&](auto et) { rc = run(et); });
+  return rc;
 }

@@ -717,9 +717,10 @@ def sparse_attention_bwd(
     pools: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ):
     """dq, dk, dv of sparse_attention_fwd (dtype of q / k / v); lse is the fp32 [B,Hq,L] tensor the forward
-    returned.  The level map carries no gradient."""
+    returned.  The level map carries no gradient.  bf16 and fp16 tensors are computed on in their own type (fp32
+    accumulation); any other type is rounded to bf16 first."""
     _require_gpu(q, k, v, level_map_, out, dout, lse)
-    qb, kb, vb, ob, dob = (_bf16_view(t) for t in (q, k, v, out, dout))
+    qb, kb, vb, ob, dob = _same_type(*(_kernel_view(t, _T16) for t in (q, k, v, out, dout)))
     B, Hq, L, D = qb.shape
     Hkv = kb.shape[1]
     sm_scale = D ** -0.5 if sm_scale is None else float(sm_scale)
@@ -731,15 +732,15 @@ def sparse_attention_bwd(
         level_map_ = level_map_.contiguous()
         if tuple(level_map_.shape) != (B, Hq, Mq, Nk):
             raise ValueError("level map must be [B, Hq, %d, %d], got %s" % (Mq, Nk, tuple(level_map_.shape)))
-        # (pools of a forward that ran in another element type are of no use to the bf16 kernels here)
-        reuse = pools is not None and pools[0] is not None and pools[0].dtype == torch.bfloat16
+        # (pools of a forward that ran in another element type are of no use to the kernels here)
+        reuse = pools is not None and pools[0] is not None and pools[0].dtype == qb.dtype
         kp, vp = pools if reuse else pool_kv(kb, vb, block_n)
     lse = lse.to(torch.float32).contiguous()
     if tuple(lse.shape) != (B, Hq, L):
         raise ValueError("lse must be [B, Hq, L]")
-    dq = torch.empty(B, Hq, L, D, dtype=torch.bfloat16, device=q.device)
-    dk = torch.empty(B, Hkv, L, D, dtype=torch.bfloat16, device=q.device)
-    dv = torch.empty(B, Hkv, L, D, dtype=torch.bfloat16, device=q.device)
+    dq = torch.empty(B, Hq, L, D, dtype=qb.dtype, device=q.device)
+    dk = torch.empty(B, Hkv, L, D, dtype=qb.dtype, device=q.device)
+    dv = torch.empty(B, Hkv, L, D, dtype=qb.dtype, device=q.device)
     ws = torch.empty(lib.psa_bwd_workspace_bytes(B, Hq, Hkv, L, D, block_n), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
         check(

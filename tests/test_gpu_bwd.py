@@ -17,11 +17,11 @@ def rel_l2(a, b):
     return float((a - b).norm() / b.norm().clamp_min(1e-30))
 
 
-def run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed, lmap=None):
+def run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed, lmap=None, dtype=torch.bfloat16):
     from psa_hip import ops
 
-    q, k, v = rnd(B, Hq, L, D, seed=seed), rnd(B, Hkv, L, D, seed=seed + 1), rnd(B, Hkv, L, D, seed=seed + 2)
-    do = rnd(B, Hq, L, D, seed=seed + 3, scale=0.5)
+    q, k, v = rnd(B, Hq, L, D, seed=seed, dtype=dtype), rnd(B, Hkv, L, D, seed=seed + 1, dtype=dtype), rnd(B, Hkv, L, D, seed=seed + 2, dtype=dtype)
+    do = rnd(B, Hq, L, D, seed=seed + 3, scale=0.5, dtype=dtype)
     Mq, Nk = -(-L // bm), -(-L // bn)
     if lmap is None:
         lmap = random_map(B, Hq, Mq, Nk, seed)
@@ -36,7 +36,8 @@ def run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed, lmap=None):
     errs = rel_l2(dq, rq), rel_l2(dk, rk), rel_l2(dv, rv)
     assert max(errs) <= REL_L2, errs
     assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
-    return dq, dk, dv, lmap
+    assert dq.dtype == dtype and dk.dtype == dtype and dv.dtype == dtype
+    return dq, dk, dv, lmap, errs
 
 
 @pytest.mark.parametrize(
@@ -68,7 +69,7 @@ def test_bwd_each_level_alone_and_unused_blocks():
     m[0, 0, 1, 2] = 8
     m[0, 1, 3, 3] = 1
     m[0, 1, 0, 0] = 2
-    dq, dk, dv, _ = run_bwd(1, 2, 2, 500, 128, 128, 128, False, seed=9, lmap=m)
+    dq, dk, dv, _, _ = run_bwd(1, 2, 2, 500, 128, 128, 128, False, seed=9, lmap=m)
     assert torch.all(dq[0, 0, :128] == 0)            # rows without keys
     assert torch.all(dk[0, 0, :256] == 0) and torch.all(dv[0, 0, :256] == 0)  # kv-blocks nobody retains
 
@@ -88,7 +89,7 @@ def test_bwd_more_than_256_rows_ordered_walks(causal):
         lmap[1, 3, 33] = 0  # ... incl. the ragged last q-block
         lmap[1, 0, :, 7] = 0  # a kv-block nobody retains
     assert B * Hq * Mq > 256
-    dq, dk, dv, _ = run_bwd(B, Hq, Hkv, L, 128, 128, 128, causal, seed=92, lmap=lmap)
+    dq, dk, dv, _, _ = run_bwd(B, Hq, Hkv, L, 128, 128, 128, causal, seed=92, lmap=lmap)
     if not causal:
         assert torch.all(dq[0, 1, 5 * 128:6 * 128] == 0) and torch.all(dq[1, 3, 33 * 128:] == 0)
 
@@ -140,3 +141,22 @@ def test_legacy_factory_autograd():
         sparse_attention_factory(128, 64, 128)
     with pytest.raises(ValueError):
         sparse_attention_factory(128, 32, 64)
+
+
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,L,D,bm,bn,causal",
+    [
+        (1, 2, 2, 600, 128, 128, 128, False),
+        (1, 4, 2, 384, 128, 128, 128, True),
+        (2, 2, 2, 500, 64, 128, 128, False),
+        (1, 2, 2, 320, 64, 64, 64, True),
+        (1, 1, 1, 400, 128, 128, 32, False),
+    ],
+)
+def test_bwd_fp16(B, Hq, Hkv, L, D, bm, bn, causal):
+    """fp16 tensors are differentiated in fp16 (fp16 MFMA operands, fp32 accumulation, gradients returned in fp16):
+    against the oracle's autograd on the fp16 values themselves, at the bound of the bf16 path - and, fp16 carrying three
+    more mantissa bits, closer to it than the bf16 run of the same case."""
+    *_, e16 = run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed=L + D, dtype=torch.float16)
+    *_, eb = run_bwd(B, Hq, Hkv, L, D, bm, bn, causal, seed=L + D, dtype=torch.bfloat16)
+    assert max(e16) <= 0.5 * max(eb), (e16, eb)
