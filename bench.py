@@ -51,16 +51,18 @@ WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.
 
 
 def fwd_traffic_bytes(workload):
-    """HBM-side bytes per launch of the forward kernel from the committed rocprofv3 counter summary
-    (profiles/psa_layer_c2_kernel_stats.txt, line `roofline.traffic <workload> <kernel> <bytes>`), or None."""
-    path = os.path.join(ROOT, "profiles", "psa_layer_c2_kernel_stats.txt")
-    try:
-        for line in open(path):
-            f = line.split()
-            if len(f) >= 4 and f[0] == "roofline.traffic" and f[1] == workload:
-                return float(f[3])
-    except OSError:
-        pass
+    """HBM-side bytes per launch of the forward kernel from the committed rocprofv3 counter summaries
+    (profiles/*.txt, line `roofline.traffic <workload> <kernel> <bytes>`), or None."""
+    import glob
+
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
+        try:
+            for line in open(path):
+                f = line.split()
+                if len(f) >= 4 and f[0] == "roofline.traffic" and f[1] == workload:
+                    return float(f[3])
+        except OSError:
+            pass
     return None
 
 
@@ -266,7 +268,7 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
         "stages_ms": stages,
         "roofline": {"kernel": "psa_fwd_pp_kernel" if (D == 128 and bm == 128) else "psa_fwd_lds_kernel", "bound": "mfma",
                      "achieved": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(fwd_flops / (t_fwd_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": fwd_traffic_bytes(args.workload),
                      "flops_per_launch": fwd_flops, "avg_launch_ms": round(t_fwd_avg, 4)},
         "cpu_baseline": cpu,
     }

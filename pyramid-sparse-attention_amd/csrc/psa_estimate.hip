@@ -257,21 +257,22 @@ __global__ __launch_bounds__(256, 2) void psa_est_gemm_lds_kernel(EstParams p) {
 // MFMA kernel (group maxima R^T [key group][query row] in log2 units, row maxima; one share of the keys).  One
 // workgroup per 64 sampled query rows; key tiles of 64 sampled keys go to LDS channel-major; thread (t / 16, t % 16)
 // owns rows ty + 16 i and keys tx + 16 j of a tile, the tile's logits pass through LDS for the group maxima.
-template <int D>
+template <int D, int RI>
 __global__ __launch_bounds__(256) void psa_est_gemm_f32_kernel(EstParams p) {
+  constexpr int QR = 16 * RI;  // sampled query rows per workgroup
   constexpr int DP = D + 1, KP = TK + 1;
   extern __shared__ __align__(16) unsigned char smem_f32[];
-  float* Qs = (float*)smem_f32;  // [64][DP]
-  float* Kt = Qs + 64 * DP;      // [D][KP]
-  float* Ss = Kt + D * KP;       // [64][KP]
+  float* Qs = (float*)smem_f32;  // [QR][DP]
+  float* Kt = Qs + QR * DP;      // [D][KP]
+  float* Ss = Kt + D * KP;       // [QR][KP]
   const float* qg = (const float*)p.q;
   const float* kg = (const float*)p.k;
   const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
   const int bh = blockIdx.y, h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
-  const int row0 = blockIdx.x * 64;
+  const int row0 = blockIdx.x * QR;
   const int32_t* oq = p.off_q ? p.off_q + (int64_t)bh * (1 << p.keep_m_log2) : nullptr;
   const int32_t* ok = p.off_k ? p.off_k + ((int64_t)b * p.Hkv + hk) * (1 << p.keep_n_log2) : nullptr;
-  for (int u = tid; u < 64 * (D / 4); u += 256) {
+  for (int u = tid; u < QR * (D / 4); u += 256) {
     const int r = u / (D / 4), c4 = u % (D / 4);
     int src = sampled_src(row0 + r, p.Ms, p.keep_m_log2, p.bm, oq, p.Lq);
     if (p.q_index != nullptr) src = clamp_row(p.q_index[src], p.Lq);
@@ -293,42 +294,42 @@ __global__ __launch_bounds__(256) void psa_est_gemm_f32_kernel(EstParams p) {
       for (int e = 0; e < 4; ++e) Kt[(c4 * 4 + e) * KP + r] = x[e];
     }
     __syncthreads();
-    float s[4][4];
+    float s[RI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < RI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) s[i][j] = 0.f;
     for (int d = 0; d < D; ++d) {
-      float qv[4], kv[4];
+      float qv[RI], kv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) qv[i] = Qs[(ty + 16 * i) * DP + d];
+      for (int i = 0; i < RI; ++i) qv[i] = Qs[(ty + 16 * i) * DP + d];
 #pragma unroll
       for (int j = 0; j < 4; ++j) kv[j] = Kt[d * KP + tx + 16 * j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < RI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[i][j] = __builtin_fmaf(qv[i], kv[j], s[i][j]);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < RI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) Ss[(ty + 16 * i) * KP + tx + 16 * j] = s[i][j] * p.qk_scale;
     __syncthreads();
     // group maxima: (row, group) pairs, row fastest so that the stores are coalesced
-    for (int u = tid; u < 64 * gpt; u += 256) {
-      const int r = u & 63, g = u >> 6;
+    for (int u = tid; u < QR * gpt; u += 256) {
+      const int r = u % QR, g = u / QR;
       float mx = -INFINITY;
       for (int c = 0; c < keep_n; ++c) mx = fmaxf(mx, Ss[r * KP + g * keep_n + c]);
       rt[(int64_t)((t0 >> p.keep_n_log2) + g) * p.Ms_pad + r] = mx;
     }
-    // row maxima: thread t < 64 keeps the maximum of row t
-    if (tid < 64) {
+    // row maxima: thread t < QR keeps the maximum of row t
+    if (tid < QR) {
       float mx = m_run;
       for (int c = 0; c < TK; ++c) mx = fmaxf(mx, Ss[tid * KP + c]);
       m_run = mx;
     }
   }
-  if (tid < 64) p.mrow[(int64_t)bh * p.Ms_pad + row0 + tid] = m_run;
+  if (tid < QR) p.mrow[(int64_t)bh * p.Ms_pad + row0 + tid] = m_run;
 }
 
 __device__ __forceinline__ float est_reduce_row(const EstParams& p, float* s_e, float* s_part, int i, int bh) {
@@ -408,10 +409,19 @@ int launch_est(EstParams& p, int B, hipStream_t stream, const LevelMapParams* lp
   grid.z = (unsigned)p.ksplit;
   if (p.dtype == PSA_DTYPE_F32) {
     p.ksplit = 1;
-    const size_t shmem = (size_t)(64 * (D + 1) + D * (TK + 1) + 64 * (TK + 1)) * sizeof(float);
-    if (hipFuncSetAttribute((const void*)psa_est_gemm_f32_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
-      return PSA_ERR_LAUNCH;
-    hipLaunchKernelGGL(psa_est_gemm_f32_kernel<D>, dim3((unsigned)(p.Ms_pad / 64), (unsigned)(B * p.Hq)), dim3(256), shmem, stream, p);
+    // 64 sampled rows per workgroup, or 32 / 16 while the launch would have fewer than two workgroups per CU
+    auto go = [&](auto ri_c) -> int {
+      constexpr int RI = decltype(ri_c)::value, QR = 16 * RI;
+      const size_t shmem = (size_t)(QR * (D + 1) + D * (TK + 1) + QR * (TK + 1)) * sizeof(float);
+      if (hipFuncSetAttribute((const void*)psa_est_gemm_f32_kernel<D, RI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+        return PSA_ERR_LAUNCH;
+      hipLaunchKernelGGL((psa_est_gemm_f32_kernel<D, RI>), dim3((unsigned)(p.Ms_pad / QR), (unsigned)(B * p.Hq)), dim3(256), shmem, stream, p);
+      return PSA_OK;
+    };
+    int ri = 4;
+    while (ri > 1 && (int64_t)(p.Ms_pad / (16 * ri)) * B * p.Hq < 512) ri >>= 1;
+    const int rc32 = ri == 4 ? go(std::integral_constant<int, 4>{}) : ri == 2 ? go(std::integral_constant<int, 2>{}) : go(std::integral_constant<int, 1>{});
+    if (rc32 != PSA_OK) return rc32;
   }
   psa_dispatch16(p.dtype, [&](auto et) {
     using ET = decltype(et);

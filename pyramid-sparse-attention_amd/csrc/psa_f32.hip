@@ -3,9 +3,11 @@
 // its Triton kernels compute in the tensors' type).  Same walk as the 16-bit kernels (psa_tiles.h: the map row is
 // compacted into tiles of 64 pooled keys of one level), same softmax (base 2, +log2(level) bias, online), same masks.
 //
-// One workgroup of 256 threads per 64 query rows (a 128-row q-block takes two workgroups).  Per tile: the K tile goes
+// One workgroup of 256 threads per QR = 16 RI query rows, RI = 4, 2 or 1 (the largest that still gives the launch two
+// workgroups per CU: the small layers this path serves would otherwise leave most of the chip idle; a 128-row q-block
+// takes 128 / QR workgroups).  Per tile: the K tile goes
 // to LDS transposed (channel-major, so that the 16 threads that share a query row read consecutive keys), the V tile
-// row-major; thread (ty, tx) = (t / 16, t % 16) owns the logits of rows ty + 16 i and keys tx + 16 j (4 x 4), reduces
+// row-major; thread (ty, tx) = (t / 16, t % 16) owns the logits of rows ty + 16 i and keys tx + 16 j (RI x 4), reduces
 // row maxima and sums over its 16-lane row group with shuffles, leaves the probabilities in LDS, and accumulates the
 // output channels tx + 16 c of its rows.  LDS-bound (two LDS operands per 16 FMAs); about 10 % of the fp32 vector peak.
 #include "psa_common.h"
@@ -13,7 +15,6 @@
 
 namespace {
 
-constexpr int QR = 64;  // query rows per workgroup
 constexpr int TK32 = 64;
 
 struct F32Params {
@@ -30,8 +31,9 @@ struct F32Params {
   const int32_t* q_index;
 };
 
-template <int D>
+template <int D, int RI>
 __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
+  constexpr int QR = 16 * RI;  // query rows per workgroup
   constexpr int DP = D + 1, KP = TK32 + 1, CPT = D / 16;  // padded strides; output channels per thread
   extern __shared__ __align__(16) unsigned char smem[];
   float* Qs = (float*)smem;         // [QR][DP]
@@ -69,10 +71,10 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
   const float* vb0 = p.v + b * p.v_sb + hk * p.v_sh;
   const int64_t BHkv = (int64_t)p.B * p.Hkv, bhk = (int64_t)b * p.Hkv + hk;
 
-  float acc[4][CPT];
-  float m_run[4], l_run[4];
+  float acc[RI][CPT];
+  float m_run[RI], l_run[RI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < RI; ++i) {
     m_run[i] = -INFINITY;
     l_run[i] = 0.f;
 #pragma unroll
@@ -100,19 +102,19 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
     }
     __syncthreads();
     // S = Q K^T: rows ty + 16 i, keys tx + 16 j
-    float s[4][4];
+    float s[RI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < RI; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) s[i][j] = 0.f;
     for (int d = 0; d < D; ++d) {
-      float qv[4], kv[4];
+      float qv[RI], kv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) qv[i] = Qs[(ty + 16 * i) * DP + d];
+      for (int i = 0; i < RI; ++i) qv[i] = Qs[(ty + 16 * i) * DP + d];
 #pragma unroll
       for (int j = 0; j < 4; ++j) kv[j] = Kt[d * KP + tx + 16 * j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < RI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[i][j] = __builtin_fmaf(qv[i], kv[j], s[i][j]);
     }
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
     for (int j = 0; j < 4; ++j) {
       const int src = s_src[tx + 16 * j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < RI; ++i) {
         const int qi = q0 + ty + 16 * i;
         const bool vis = src >= 0 && (!p.causal || (((int64_t)src + 1) << tr.lv) - 1 <= qi);
         s[i][j] = vis ? __builtin_fmaf(s[i][j], p.scale_log2, bias) : -INFINITY;
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
     }
     // online softmax per row over the 16 lanes of the row group
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < RI; ++i) {
       float mx = fmaxf(fmaxf(s[i][0], s[i][1]), fmaxf(s[i][2], s[i][3]));
       for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
       const float m_new = fmaxf(m_run[i], mx);
@@ -152,19 +154,19 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
     __syncthreads();
     // O += P V: rows ty + 16 i, channels tx + 16 c
     for (int kk = 0; kk < TK32; ++kk) {
-      float pv[4], vv[CPT];
+      float pv[RI], vv[CPT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pv[i] = Ps[(ty + 16 * i) * KP + kk];
+      for (int i = 0; i < RI; ++i) pv[i] = Ps[(ty + 16 * i) * KP + kk];
 #pragma unroll
       for (int c = 0; c < CPT; ++c) vv[c] = Vs[kk * D + tx + 16 * c];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < RI; ++i)
 #pragma unroll
         for (int c = 0; c < CPT; ++c) acc[i][c] = __builtin_fmaf(pv[i], vv[c], acc[i][c]);
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < RI; ++i) {
     const int qi = q0 + ty + 16 * i;
     if (qi >= p.L || qi >= (I + 1) * p.bm) continue;
     const int orow = p.q_index != nullptr ? p.q_index[qi] : qi;
@@ -178,15 +180,16 @@ __global__ __launch_bounds__(256) void psa_fwd_f32_kernel(F32Params p) {
   }
 }
 
-template <int D>
+template <int D, int RI>
 int launch_f32(const F32Params& p, hipStream_t stream) {
+  constexpr int QR = 16 * RI;
   const size_t shmem = (size_t)(QR * (D + 1) + D * (TK32 + 1) + TK32 * D + QR * (TK32 + 1)) * 4 + TK32 * 4 + (size_t)p.max_tiles * 8 +
                        (size_t)p.Nk * 2 + 16;
   if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
-  if (hipFuncSetAttribute((const void*)psa_fwd_f32_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+  if (hipFuncSetAttribute((const void*)psa_fwd_f32_kernel<D, RI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
     return PSA_ERR_LAUNCH;
   const int64_t units = (int64_t)p.B * p.Hq * p.Mq * p.halves;
-  hipLaunchKernelGGL(psa_fwd_f32_kernel<D>, dim3((unsigned)units), dim3(256), shmem, stream, p);
+  hipLaunchKernelGGL((psa_fwd_f32_kernel<D, RI>), dim3((unsigned)units), dim3(256), shmem, stream, p);
   return PSA_OK;
 }
 
@@ -209,7 +212,7 @@ int psa_fwd_f32(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
                 PSA_ERR_UNSUPPORTED, "psa_fwd: fp32 tensors must be 16-byte aligned with strides that are multiples of 4 elements");
   const int Mq = (L + block_m - 1) / block_m, Nk = (L + block_n - 1) / block_n;
   PSA_REQUIRE(Nk <= 65535, PSA_ERR_UNSUPPORTED, "psa_fwd: more than 65535 kv-blocks");
-  PSA_REQUIRE((int64_t)B * Hq * Mq * 2 < (1ll << 31), PSA_ERR_UNSUPPORTED, "psa_fwd: too many workgroups");
+  PSA_REQUIRE((int64_t)B * Hq * Mq * 8 < (1ll << 31), PSA_ERR_UNSUPPORTED, "psa_fwd: too many workgroups");
   F32Params p;
   p.q = (const float*)q.ptr; p.k = (const float*)k.ptr; p.v = (const float*)v.ptr; p.o = (float*)out.ptr;
   p.kp = (const float*)k_pool; p.vp = (const float*)v_pool;
@@ -219,13 +222,19 @@ int psa_fwd_f32(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_pool,
   p.v_sb = v.stride_b; p.v_sh = v.stride_h; p.v_sl = v.stride_l;
   p.o_sb = out.stride_b; p.o_sh = out.stride_h; p.o_sl = out.stride_l;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.L = L; p.Mq = Mq; p.Nk = Nk;
-  p.bn_log2 = psa_ilog2(block_n); p.bm = block_m; p.halves = block_m / QR;
+  // rows per workgroup: 64, or 32 / 16 while the launch would have fewer than two workgroups per CU
+  int ri = 4;
+  while (ri > 1 && (int64_t)B * Hq * Mq * (block_m / (16 * ri)) < 512) ri >>= 1;
+  p.bn_log2 = psa_ilog2(block_n); p.bm = block_m; p.halves = block_m / (16 * ri);
   p.npad = (int64_t)Nk * block_n;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
   p.causal = causal ? 1 : 0;
   p.max_tiles = (block_n >= 64 ? Nk * (block_n / 64) : (Nk * block_n + 63) / 64) + 4;
   p.q_index = q_index;
-  const int rc = D == 128 ? launch_f32<128>(p, (hipStream_t)stream) : launch_f32<64>(p, (hipStream_t)stream);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (D == 128) rc = ri == 4 ? launch_f32<128, 4>(p, st) : ri == 2 ? launch_f32<128, 2>(p, st) : launch_f32<128, 1>(p, st);
+  else rc = ri == 4 ? launch_f32<64, 4>(p, st) : ri == 2 ? launch_f32<64, 2>(p, st) : launch_f32<64, 1>(p, st);
   PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the fp32 kernel's on-chip schedule (LDS)");
   return psa_check_launch("psa_fwd (fp32)");
 }

@@ -13,6 +13,7 @@ namespace psa_order {
 namespace {  // one private copy per translation unit that launches them
 
 constexpr int COST_BINS = 2048;
+constexpr int SMALL_CHUNK = 512;  // shares up to this many items are ordered by rank counting in one pass
 constexpr int MAX_PHASES = 64;
 constexpr int64_t PHASE_BYTES = 128ll << 20;  // operand bytes (K/V + pooled levels, or Q/dO) in use at one time
 
@@ -61,6 +62,27 @@ __global__ __launch_bounds__(256) void psa_chunk_sort_kernel(const int32_t* cost
   __shared__ int hist[COST_BINS];
   const int x = blockIdx.x, tid = threadIdx.x;
   const int r0 = x * chunk;
+  if (chunk <= SMALL_CHUNK) {
+    // short shares (the usual case): the slot of an item is its rank among the keys (decreasing cost, then index) -
+    // the same stable order as the counting sort below, without histogram, scan and their barriers
+    __shared__ __attribute__((aligned(16))) uint32_t keys[SMALL_CHUNK];
+    for (int i = tid; i < SMALL_CHUNK; i += 256)
+      keys[i] = i < chunk && r0 + i < total ? ((uint32_t)(COST_BINS - 1 - cost[r0 + i]) << 16) | (uint32_t)i : 0xffffffffu;
+    __syncthreads();
+    const int n4 = (chunk + 3) >> 2;
+    for (int i = tid; i < chunk; i += 256) {
+      const uint32_t mine = keys[i];
+      int rank = 0;
+      for (int j = 0; j < n4; ++j) {
+        const u32x4 k4 = ((const u32x4*)keys)[j];
+        rank += (k4[0] < mine) + (k4[1] < mine) + (k4[2] < mine) + (k4[3] < mine);
+      }
+      if (mine != 0xffffffffu) order[r0 + rank] = r0 + i;
+    }
+    const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;
+    for (int i = valid + tid; i < chunk; i += 256) order[r0 + i] = -1;
+    return;
+  }
   for (int i = tid; i < COST_BINS; i += 256) hist[i] = 0;
   __syncthreads();
   for (int i = tid; i < chunk; i += 256)
