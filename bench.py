@@ -382,6 +382,9 @@ def main():
     it = max(10, min(args.steps, 100))
     t_pool, _ = time_gpu(lambda: ops.pool_kv(k, v, bn), it)
     t_est, _ = time_gpu(lambda: ops.estimate_sampled(q, k, off_q, off_k, bm, bn, km, kn), it)
+    # the sampling offsets of a layer call (one device-side draw for q and k; the timed layer takes fixed offsets so
+    # that every step computes the same map)
+    t_draw, _ = time_gpu(lambda: ops.draw_sample_offsets(B, H, H, bm, km, bn, kn, dev), it)
     t_map, _ = time_gpu(lambda: ops.level_map(state["s"], ratios, text, mode, blocksize=bn, compute_tile=tn, map_dtype=torch.int8), it)
     out_buf = torch.empty_like(q)
     # the map's tile schedule is built once per map (by the layer, right after the map): timed as a stage of its own,
@@ -541,7 +544,7 @@ def main():
         "data": "synthetic (seeded smooth 3-D field + noise, logit std ~3)",
         "config": {"workload": w["name"], "L": L, "block_m": bm, "block_n": bn, "density": round(density, 4),
                    "sparsity": round(1 - density, 4), "mask_mode": mode, "tau": None if tau != tau else round(tau, 4)},
-        "stages_ms": {"pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
+        "stages_ms": {"sampling_draw": round(t_draw, 4), "pool": round(t_pool, 4), "estimate": round(t_est, 4), "level_map": round(t_map, 4),
                       "schedule": None if t_sched is None else round(t_sched, 4), "sparse_fwd": round(t_fwd_med, 4), "layer": round(ms_step, 4), "wall_per_step": round(wall_ms / args.steps, 4),
                       "layer_graph": round(t_graph, 4), "layer_graph_bit_identical": graph_equal},
         "reorder_ms": reorder,

@@ -12,7 +12,9 @@
 namespace psa_order {
 namespace {  // one private copy per translation unit that launches them
 
-constexpr int COST_BINS = 2048;
+constexpr int COST_BINS = 2048, COST_BITS = 11;
+static_assert(COST_BINS == 1 << COST_BITS, "cost bins");
+constexpr int RADIX_IPT = 16, RADIX_CHUNK = 256 * RADIX_IPT;  // shares up to this many items are radix-sorted in LDS
 constexpr int SMALL_CHUNK = 512;  // shares up to this many items are ordered by rank counting in one pass
 constexpr int MAX_PHASES = 64;
 constexpr int64_t PHASE_BYTES = 128ll << 20;  // operand bytes (K/V + pooled levels, or Q/dO) in use at one time
@@ -81,6 +83,59 @@ __global__ __launch_bounds__(256) void psa_chunk_sort_kernel(const int32_t* cost
     }
     const int valid = total - r0 < chunk ? (total - r0 > 0 ? total - r0 : 0) : chunk;
     for (int i = valid + tid; i < chunk; i += 256) order[r0 + i] = -1;
+    return;
+  }
+  if (chunk <= RADIX_CHUNK) {
+    // medium shares: stable binary radix sort (least significant bit first) on the inverted cost, one bit per pass; a
+    // thread owns a run of consecutive items, so "earlier" is (earlier thread, then earlier in the run)
+    __shared__ uint32_t kbuf[2][RADIX_CHUNK];
+    __shared__ int wave_tot[4];
+    const int ipt = (chunk + 255) >> 8;  // items per thread (<= RADIX_IPT)
+    const int i0 = tid * ipt;
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < chunk; i += 256)
+      kbuf[0][i] = r0 + i < total ? ((uint32_t)(COST_BINS - 1 - cost[r0 + i]) << 16) | (uint32_t)i : 0xffffffffu;
+    __syncthreads();
+    int src = 0;
+    for (int bit = 16; bit < 16 + COST_BITS; ++bit) {
+      uint32_t k[RADIX_IPT];
+      int zeros = 0;
+#pragma unroll
+      for (int e = 0; e < RADIX_IPT; ++e) {
+        k[e] = (e < ipt && i0 + e < chunk) ? kbuf[src][i0 + e] : 0xffffffffu;
+        zeros += (e < ipt && i0 + e < chunk && !((k[e] >> bit) & 1u)) ? 1 : 0;
+      }
+      // exclusive scan of the zero counts over the 256 threads
+      int incl = zeros;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        incl += lane >= d ? up : 0;
+      }
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      int before = incl - zeros, all_zeros = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        before += w < wave ? wave_tot[w] : 0;
+        all_zeros += wave_tot[w];
+      }
+      int z = before, o = all_zeros + (i0 < chunk ? i0 : chunk) - before;  // next slot of a zero / of a one
+#pragma unroll
+      for (int e = 0; e < RADIX_IPT; ++e)
+        if (e < ipt && i0 + e < chunk) {
+          const bool one = (k[e] >> bit) & 1u;
+          kbuf[src ^ 1][one ? o : z] = k[e];
+          o += one ? 1 : 0;
+          z += one ? 0 : 1;
+        }
+      __syncthreads();
+      src ^= 1;
+    }
+    for (int i = tid; i < chunk; i += 256) {
+      const uint32_t key = kbuf[src][i];
+      order[r0 + i] = key != 0xffffffffu ? r0 + (int)(key & 0xffffu) : -1;
+    }
     return;
   }
   for (int i = tid; i < COST_BINS; i += 256) hist[i] = 0;

@@ -89,3 +89,47 @@ def test_strided_rows_fall_back_to_the_map_walk():
     o1 = ops.sparse_attention_fwd(q, kt, vt, lmap, BM, BN)
     torch.cuda.synchronize()
     assert kt.stride(2) != D and torch.equal(o0, o1)
+
+
+@pytest.mark.parametrize("H,Hkv,L", [(3, 3, 128 * 40), (40, 1, 128 * 128), (64, 1, 128 * 300 + 5), (160, 1, 128 * 300)])
+def test_issue_order_is_a_stable_sort_of_every_share(H, Hkv, L):
+    """The schedule's issue order (layout: 64 bytes | order | cost | tiles | records of 2 Nk + 4 entries of 16 bytes, every
+    part padded to 64 bytes): a permutation of the rows in equal shares, each share sorted by decreasing tile count
+    with equal counts in index order - for shares of 15 rows (rank counting), 640 and 2408 (radix sort in LDS) and 6020
+    (counting sort)."""
+    from psa_hip import ops
+
+    B = 1
+    Mq = Nk = -(-L // BM)
+    rows = B * H * Mq
+    g = torch.Generator().manual_seed(H)
+    keep = torch.rand(B, H, Mq, 1, generator=g) ** 2  # strongly uneven rows, many ties among the short ones
+    lmap = torch.from_numpy(random_map(B, H, Mq, Nk, 5, ensure_row=False))
+    lmap = torch.where(torch.rand(B, H, Mq, Nk, generator=g) < keep, lmap, torch.zeros_like(lmap)).to(torch.int8).to(dev())
+    from psa_hip._lib import lib
+
+    buf = torch.full((lib.psa_schedule_bytes(B, H, Hkv, L, D, BM, BN),), 0x5A, dtype=torch.uint8, device=dev())
+    sched = ops.build_schedule(lmap, Hkv, L, D, BM, BN, out=buf)
+    torch.cuda.synchronize()
+    words = sched.cpu().view(torch.int32)
+    rows_pad = -(-rows // 16) * 16  # every part is padded to 64 bytes
+    n_pad = (words.numel() * 4 - 64 - rows_pad * 8 - rows * (2 * Nk + 4) * 16) // 4
+    order = words[16:16 + n_pad].numpy()
+    while order[-1] == 0x5A5A5A5A:  # the padding behind the last share is never written
+        order = order[:-1]
+    n_order = len(order)
+    tiles = words[16 + n_pad + rows_pad:16 + n_pad + rows_pad + rows].numpy().astype(np.int64)
+    live = order[order >= 0]
+    assert np.array_equal(np.sort(live), np.arange(rows))
+    t = np.where(order >= 0, tiles[np.clip(order, 0, rows - 1)], -1)
+    key_a = t[:-1] * (1 << 32) - order[:-1]   # decreasing tiles, then increasing index (pads: -1 tiles, last)
+    key_b = t[1:] * (1 << 32) - order[1:]
+    breaks = np.nonzero((key_b > key_a) & (order[1:] >= 0))[0] + 1  # where a new share starts
+    assert len(breaks) > 0
+    chunk = int(np.gcd.reduce(np.append(breaks, n_order)))
+    assert n_order % chunk == 0 and (n_order // chunk) % 8 == 0, (chunk, n_order)
+    for s0 in range(0, n_order, chunk):
+        share = order[s0:s0 + chunk]
+        share = share[share >= 0]
+        want = sorted(share.tolist(), key=lambda r: (-min(int(tiles[r]), 2047), r))
+        assert share.tolist() == want, s0
