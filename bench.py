@@ -398,8 +398,8 @@ def main():
     sclk = None if args.no_extras else sclk_under_load(fwd_call, t_fwd_avg)
     t_dense = t_sdpa = None
     if not args.no_dense:
-        t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=1)
-        t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=1)
+        t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=5)
+        t_sdpa, _ = time_gpu(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), max(3, it // 10), warm=3)
 
     reorder = preset = None
     if not args.no_extras:

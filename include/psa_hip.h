@@ -12,8 +12,9 @@
  *   - work is enqueued on `stream` (a hipStream_t passed as void*), no host synchronisation;
  *   - return value 0 = ok, negative = error (see PSA_ERR_*); psa_last_error() gives a
  *     thread-local human-readable message for the last failing call on this thread;
- *   - activations are bf16, [B, H, L, D] with the D axis contiguous; batch/head/row strides are
- *     given in elements (psa_tensor4), so transposed [B, L, H, D] views need no copy;
+ *   - activations are bf16, fp16 or fp32 (psa_tensor4.dtype; see PSA_DTYPE_* for which entry points take which),
+ *     [B, H, L, D] with the D axis contiguous; batch/head/row strides are given in elements (psa_tensor4), so
+ *     transposed [B, L, H, D] views need no copy;
  *   - D in {64, 128}; block_m in {64, 128}; block_n in {32, 64, 128};
  *   - level maps hold one of {0, 1, 2, 4, 8} per (q-block, kv-block): 0 = skip, l = attend to the
  *     kv-block's keys mean-pooled by l.  `map_elem_bytes` is 1 (int8) or 4 (int32, the reference's
@@ -43,7 +44,9 @@ typedef void* psa_stream_t; /* hipStream_t */
 /* Element types.  The kernels compute in the type of their tensors, as the reference's do (tl.dot on q / k as loaded,
  * p.to(v.dtype): reference src/psa_triton/kernels/psa_kernel.py:49-77): bf16 and fp16 operands on the matrix cores with
  * fp32 accumulation, fp32 tensors in fp32 throughout.  All tensors of one call (and its pooled buffers) share one
- * type.  Entry points say which types they take; the others return PSA_ERR_UNSUPPORTED. */
+ * type.  bf16 and fp16: every entry point that takes tensors, except psa_estimate_xattn (bf16 only).  fp32: psa_pool_kv*,
+ * psa_estimate_sampled* and the psa_fwd* family (vector-unit kernels; psa_build_schedule / psa_fwd_scheduled are for the
+ * 16-bit types); psa_bwd, psa_ksim and psa_estimate_xattn return PSA_ERR_UNSUPPORTED for fp32 tensors. */
 #define PSA_DTYPE_BF16 0
 #define PSA_DTYPE_F16 1
 #define PSA_DTYPE_F32 2
@@ -61,14 +64,14 @@ typedef struct psa_tensor4 {
 int psa_version(void);
 const char* psa_last_error(void);
 
-/* Number of bf16 elements of one pooled buffer (levels 2, 4, 8 back to back):
+/* Number of elements (of the tensors' type) of one pooled buffer (levels 2, 4, 8 back to back):
  * B*Hkv*Npad*D*7/8 with Npad = ceil(L/block_n)*block_n.  Level l starts at element
  * psa_pool_level_offset(...) and is a contiguous [B, Hkv, Npad/l, D]. */
 int64_t psa_pool_elems(int B, int Hkv, int L, int D, int block_n);
 int64_t psa_pool_level_offset(int B, int Hkv, int L, int D, int block_n, int level);
 
 /* Pyramid pooling of K and V: one pass that reads K, V once and writes the 2x, 4x, 8x mean-pooled
- * levels (each level rounded to bf16 before the next, tail replicate-padded to block_n).
+ * levels (each level rounded to the tensors' type before the next, tail replicate-padded to block_n).
  * Replaces pad_to_multiple + pooling x3 per tensor:
  *   reference src/psa_triton/kernels/psa_kernel.py:318-349,381-388
  *   (same code at src/psa_triton/kernels/psa_kernel_legacy.py:806-834,868-875). */
@@ -230,7 +233,7 @@ int psa_fwd_indexed(psa_tensor4 q, const int32_t* q_index, psa_tensor4 k, psa_te
 int psa_density(const void* map, int map_elem_bytes, int64_t bh, int Mq, int Nk, int causal,
                 float* density_out, psa_stream_t stream);
 
-/* Sparse attention forward from a level map.  out [B, Hq, L, D] bf16; lse (may be NULL)
+/* Sparse attention forward from a level map.  out [B, Hq, L, D] in the type of q / k / v (bf16, fp16 or fp32); lse (may be NULL)
  * [B, Hq, L] fp32 = natural-log softmax denominator incl. the +ln(level) bias; map == NULL means
  * dense attention (every pair at level 1; k_pool/v_pool may then be NULL).  K/V have Hkv heads,
  * query head h uses kv head h / (Hq/Hkv).  causal != 0: kv-blocks above the diagonal are never
@@ -292,8 +295,8 @@ int64_t psa_fwd_noalloc_max_rows(void);
  * the dQ rows and of the dK/dV workgroups). */
 int64_t psa_bwd_workspace_bytes(int B, int Hq, int Hkv, int L, int D, int block_n);
 
-/* Backward of psa_fwd w.r.t. q, k, v (the map carries no gradient).  dq/dk/dv are bf16 views like
- * q/k/v; workspace is caller-allocated (psa_bwd_workspace_bytes) and is overwritten.
+/* Backward of psa_fwd w.r.t. q, k, v (the map carries no gradient).  bf16 or fp16 tensors; dq/dk/dv are views like
+ * q/k/v in the same type; workspace is caller-allocated (psa_bwd_workspace_bytes) and is overwritten.
  * Gradients of pooled keys are spread over their constituent tokens (/level) and the part that
  * lands on replicate-pad positions is added to the last real token.
  * Replaces _sparse_attention.backward and its kernels:

@@ -324,6 +324,8 @@ extern "C" int psa_estimate_xattn(psa_tensor4 q, psa_tensor4 k, float* est, void
                   q.stride_h % 8 == 0 && k.stride_h % 8 == 0 && q.stride_b % 8 == 0 && k.stride_b % 8 == 0,
               PSA_ERR_UNSUPPORTED, "psa_estimate_xattn: tensors must be 16-byte aligned with strides multiple of 8");
   PSA_REQUIRE((int64_t)B * Hq <= 65535, PSA_ERR_UNSUPPORTED, "psa_estimate_xattn: B*Hq too large");
+  PSA_REQUIRE(q.dtype == PSA_DTYPE_BF16 && k.dtype == PSA_DTYPE_BF16, PSA_ERR_UNSUPPORTED,
+              "psa_estimate_xattn: bf16 tensors only (element type %d / %d)", q.dtype, k.dtype);
   const XGeom g = xgeom(Lq, Lk, block_size, stride, chunk_size);
   XParams p;
   p.q = (const bf16_t*)q.ptr; p.k = (const bf16_t*)k.ptr;

@@ -658,8 +658,8 @@ def psa_layer_fwd_graph(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, off_q
                         mode: str, block_m: int, block_n: int, tile_n: int, **kwargs):
     """psa_layer_fwd captured into one HIP graph and replayed: the estimator, the reduction + level map, the tile schedule
     and the attention kernel on the main branch, the pooling pass on a second branch beside the estimator - kernel nodes
-    only (the library enqueues nothing else: no memset or copy nodes), so the launch gaps and the stream fork / join of
-    the eager sequence disappear.  The graph is tied to the ADDRESSES of q, k, v and the offsets (and to every other
+    only (the library enqueues nothing else: no memset or copy nodes).  For callers that replay graphs anyway; on its own it
+    is no faster than the eager operator, whose launches are enqueued far ahead of the GPU.  The graph is tied to the ADDRESSES of q, k, v and the offsets (and to every other
     argument): a call with tensors at the same addresses replays it on their current contents, any other call captures
     a new graph (a few are kept).  The returned tensors belong to the graph and are overwritten by its next replay.
     Same bits as psa_layer_fwd.  Keyword arguments as psa_layer_fwd (tensors among them are part of the key)."""
