@@ -396,6 +396,18 @@ def main():
     fwd_call = lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf, schedule=sched)
     t_fwd_med, t_fwd_avg = time_gpu(fwd_call, it)
     sclk = None if args.no_extras else sclk_under_load(fwd_call, t_fwd_avg)
+    lib_gemm = None
+    if not args.no_extras:
+        # context: what the vendor library's bf16 GEMM (torch.matmul, 8192^3) sustains on this box, and at which clock
+        ga = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        gb = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        gemm_call = lambda: torch.matmul(ga, gb)
+        _, t_gemm = time_gpu(gemm_call, 30)
+        lib_gemm = {"what": "torch.matmul bf16 8192 x 8192 x 8192", "ms": round(t_gemm, 4),
+                    "tflops": round(2.0 * 8192 ** 3 / (t_gemm * 1e-3) / 1e12, 1),
+                    "frac_of_peak": round(2.0 * 8192 ** 3 / (t_gemm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+                    "sclk_mhz_under_load": sclk_under_load(gemm_call, t_gemm)}
+        del ga, gb
     t_dense = t_sdpa = None
     if not args.no_dense:
         t_dense, _ = time_gpu(lambda: ops.sparse_attention_fwd(q, k, v, None, bm, bn, out=out_buf), max(3, it // 10), warm=5)
@@ -549,6 +561,7 @@ def main():
                       "layer_graph": round(t_graph, 4), "layer_graph_bit_identical": graph_equal},
         "reorder_ms": reorder,
         "preset_ms": preset,
+        "library_gemm": lib_gemm,
         "executed_tflops_fwd": round(exec_flops / (t_fwd_med * 1e-3) / 1e12, 2),
         "pct_bf16_peak_fwd_executed": round(100 * exec_flops / (t_fwd_med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
         "pool_gbs": round(pool_bytes / (t_pool * 1e-3) / 1e9, 1),
