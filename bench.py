@@ -1,10 +1,10 @@
 """Benchmark of the PSA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5] [--no-cpu] [--no-dense] [--no-extras]
 
 A step = one PSA attention layer over synthetic inputs already resident in HBM:
-pyramid pooling -> sampled block-importance estimate -> level map -> sparse attention forward.
-Prints ONE JSON line (metric of BASELINE.json) with a `roofline` object for the dominant kernel
+pyramid pooling -> sampled block-importance estimate -> level map -> tile schedule -> sparse attention forward.
+Prints ONE JSON line (the headline metric of this path) with a `roofline` object for the dominant kernel
 (the sparse forward, MFMA-bound) and a `cpu_baseline` object (the oracle on the host cores over a
 bounded sample of the same workload).
 """
@@ -25,24 +25,24 @@ PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
-    # BASELINE.json configs[1]: Wan2.1-1.3B 480p self-attention layer
+    # c2, the configuration the metric is quoted on: Wan2.1-1.3B 480p self-attention layer
     "c2": dict(name="wan2.1-1.3b-480p B1 H12 N32760 D128 bf16 blk128 thresholdbound ~90% sparsity",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.90),
-    # BASELINE.json configs[0] (small, fp32 tensors: every stage computes in fp32 - the fp32 kernels run on the vector
+    # c1 (small, fp32 tensors: every stage computes in fp32 - the fp32 kernels run on the vector
     # units, so the peak its roofline line is priced against is the fp32 one)
     "c1": dict(name="small B1 H2 N4096 D64 fp32 blk64 thresholdbound ~80% sparsity",
                B=1, H=2, grid=(4, 32, 32), D=64, bm=64, bn=64, tn=16, sparsity=0.80, dtype="fp32"),
 }
 WORKLOADS.update({
-    # BASELINE.json configs[2]: CogVideoX-5B joint text + video attention (text blocks last, always level 1)
+    # c3: CogVideoX-5B joint text + video attention (text blocks last, always level 1)
     # (top-k with the ratios of the reference's CogVideo_5b / psa_4steps preset: density 0.15625 before the text columns)
     "c3": dict(name="cogvideox-5b B2 H48 N17776 (17550 video + 226 text) D64 bf16 blk128 topk psa_4steps ratios ~84% sparsity",
                B=2, H=48, grid=(13, 30, 45), D=64, bm=128, bn=128, tn=32, sparsity=0.84, text=226, mode="topk",
                ratios={1: (0.0, 0.05), 2: (0.05, 0.15), 4: (0.15, 0.25), 8: (0.25, 0.5), 0: (0.5, 1.0)}),
-    # BASELINE.json configs[3]: training step = forward with lse + backward (dQ, dK, dV)
+    # c4: training step = forward with lse + backward (dQ, dK, dV)
     "c4": dict(name="training step B1 H12 N32760 D128 bf16 blk128 thresholdbound ~85% sparsity, dO ~ N(0, 0.02)",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.85, kind="train"),
-    # BASELINE.json configs[4]: causal GQA prefill at the Qwen2.5-VL-7B decoder shape
+    # c5: causal GQA prefill at the Qwen2.5-VL-7B decoder shape
     "c5": dict(name="qwen2.5-vl-7b causal prefill B1 Hq28 Hkv4 N32768 (1024 text + 16x44x44 vision) D128 bf16 blk128 "
                     "xattn estimate stride 8, energybound ~80% sparsity over the lower triangle",
                B=1, H=28, Hkv=4, grid=(16, 44, 44), D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal", stride=8),
