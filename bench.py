@@ -43,9 +43,12 @@ WORKLOADS.update({
     "c4": dict(name="training step B1 H12 N32760 D128 bf16 blk128 thresholdbound ~85% sparsity, dO ~ N(0, 0.02)",
                B=1, H=12, grid=(21, 30, 52), D=128, bm=128, bn=128, tn=32, sparsity=0.85, kind="train"),
     # c5: causal GQA prefill at the Qwen2.5-VL-7B decoder shape
-    "c5": dict(name="qwen2.5-vl-7b causal prefill B1 Hq28 Hkv4 N32768 (1024 text + 16x44x44 vision) D128 bf16 blk128 "
-                    "xattn estimate stride 8, energybound ~80% sparsity over the lower triangle",
-               B=1, H=28, Hkv=4, grid=(16, 44, 44), D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal", stride=8),
+    # (the configuration names N = 32768 with tokens 1024.. on a 16x44x44 grid, which has 30976 positions: the vision
+    # part here is the first 31744 positions of a 17x44x44 grid, so that N is the 32768 the configuration is about)
+    "c5": dict(name="qwen2.5-vl-7b causal prefill B1 Hq28 Hkv4 N32768 (1024 text + 31744 vision tokens of a 44x44-per-frame grid) "
+                    "D128 bf16 blk128 xattn estimate stride 8, energybound ~80% sparsity over the lower triangle",
+               B=1, H=28, Hkv=4, grid=(17, 44, 44), tokens=32768, D=128, bm=128, bn=128, sparsity=0.80, text=1024, kind="causal",
+               stride=8),
 })
 WAN13 = {1: (0.0, 0.5), 2: (0.5, 0.6), 4: (0.6, 0.7), 8: (0.7, 0.8), 0: (0.8, 1.0)}
 
@@ -186,6 +189,8 @@ def run_other(args, w, torch, ops, make_qkv, sample_offsets, dev):
     text = w.get("text", 0)
     causal = w["kind"] == "causal"
     q, k, v = make_qkv(B, H, Hkv, w["grid"], D, seed=args.seed, device=dev, text_tokens=text, text_first=causal)
+    if "tokens" in w:
+        q, k, v = (t[:, :, :w["tokens"]].contiguous() for t in (q, k, v))
     L = q.shape[2]
     it = max(5, min(args.steps, 30))
     stages = {}

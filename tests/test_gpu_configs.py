@@ -186,6 +186,36 @@ def test_c3_cogvideox_reduced_end_to_end_vs_oracle():
     assert np.array_equal(mask.cpu().numpy(), O.level_map(scores.cpu().numpy(), COG_4STEPS, 0, "topk", blocksize=bn, compute_tile=tn))
 
 
+def test_c3_cogvideox_full_size_vs_oracle():
+    """The CogVideoX-5B configuration at its own size: B 2, H 48, N 17776 (13x30x45 video grid + 226 text tokens), D 64,
+    blocks of 128, top-k with the preset's ratios, the layer operator (head dim 64: the one-row kernel).  Scores of four
+    (batch, head) pairs against the oracle (rtol 2e-4), their map rows bit for bit from the GPU's scores (text columns at
+    level 1), and their outputs - all q-blocks - against the oracle's block walk (max-abs 2e-2, mean-abs 2e-3)."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    B, H, D, bm, bn, tn, text = 2, 48, 64, 128, 128, 32, 226
+    q, k, v = make_qkv(B, H, H, (13, 30, 45), D, seed=1234, text_tokens=text)
+    L = q.shape[2]
+    assert L == 17776
+    oq, ok = sample_offsets(B, H, bm, 32, 1244), sample_offsets(B, H, bn, 32, 1245)
+    qd, kd, vd, oqd, okd = (t.to(dev()) for t in (q, k, v, oq, ok))
+    out, mp = ops.psa_layer_fwd(qd, kd, vd, oqd, okd, COG_4STEPS, "topk", bm, bn, tn, return_map=True, text_length=text)
+    scores = ops.estimate_sampled(qd, kd, oqd, okd, bm, bn, 32, 32)
+    torch.cuda.synchronize()
+    torch.set_num_threads(min(torch.get_num_threads(), 16))
+    heads = [0, 47]
+    ref_scores = O.estimate_sampled(q[:, heads], k[:, heads], bm, bn, oq[:, heads], ok[:, heads])
+    np.testing.assert_allclose(scores[:, heads].cpu().numpy(), ref_scores.numpy(), rtol=2e-4, atol=1e-9)
+    ref_map = O.level_map(scores[:, heads].cpu().numpy(), COG_4STEPS, text, "topk", blocksize=bn, compute_tile=tn)
+    got_map = mp[:, heads].cpu().numpy()
+    assert np.array_equal(got_map, ref_map)
+    assert (got_map[..., -2:] == 1).all()
+    ref, _ = O.psa_attention_blockwalk(q[:, heads], k[:, heads], v[:, heads], ref_map, bm, bn)
+    mx, mean = attn_errors(out[:, heads], ref)
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+
+
 def test_c3_kernel_at_full_length_lossless_property():
     """The kernel c3 runs (head dim 64, 128-row q-blocks: the one-row kernel) at c3's sequence length N = 17776
     (139 blocks, last one 112 tokens), one head, random map without skips on group-constant K/V vs SDPA."""
@@ -292,6 +322,39 @@ def test_c5_reduced_prefill_vs_oracle():
     ref, _ = O.psa_attention_blockwalk(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), ref_map, 128, 128, causal=True)
     mx, mean = attn_errors(out, ref)
     assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+
+
+def test_c5_qwen_prefill_full_size_vs_oracle():
+    """The causal prefill configuration at its own size: B 1, 28 query heads on 4 kv heads, N 32768 (1024 text tokens first,
+    then the first 31744 positions of a 17x44x44 vision grid), D 128, antidiagonal estimate at stride 8, energy-bound map, causal GQA forward through the
+    tile schedule.  For the first and the last query head: estimate against the oracle, map rows bit for bit from the
+    GPU's estimate, output and LSE of every q-block against the oracle's causal block walk."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv
+
+    B, Hq, Hkv, D, text = 1, 28, 4, 128, 1024
+    q, k, v = (t[:, :, :32768].contiguous() for t in make_qkv(B, Hq, Hkv, (17, 44, 44), D, seed=1234, text_tokens=text, text_first=True))
+    L = q.shape[2]
+    assert L == 32768
+    ratios = {1: (0.0, 0.3), 2: (0.3, 0.36), 4: (0.36, 0.42), 8: (0.42, 0.48), 0: (0.48, 1.0)}
+    qd, kd, vd = q.to(dev()), k.to(dev()), v.to(dev())
+    est = ops.estimate_xattn(qd, kd, block_size=128, stride=8, causal=True)
+    mp = ops.level_map_qwen(est, ratios, text, "energybound", block_size=128, causal=True, map_dtype=torch.int8)
+    out, lse, _ = ops.sparse_attention_fwd(qd, kd, vd, mp, 128, 128, causal=True, return_lse=True)
+    torch.cuda.synchronize()
+    dens = float(ops.density(mp, causal=True)[-1])
+    assert 0.05 < dens < 0.6, dens
+    torch.set_num_threads(min(torch.get_num_threads(), 16))
+    for h in (0, 27):
+        hk = h // (Hq // Hkv)
+        ref_est = O.estimate_xattn(q[:, h:h + 1].float(), k[:, hk:hk + 1].float(), 128, 8, True)
+        np.testing.assert_allclose(est[:, h:h + 1].cpu().numpy(), ref_est.numpy(), rtol=2e-3, atol=2e-6)
+        ref_map = O.level_map_qwen(est[:, h:h + 1].cpu().numpy(), ratios, text_length=text, mode="energybound", block_size=128, causal=True)
+        assert np.array_equal(mp[:, h:h + 1].cpu().numpy(), ref_map)
+        ref, ref_lse = O.psa_attention_blockwalk(q[:, h:h + 1], k[:, hk:hk + 1], v[:, hk:hk + 1], ref_map, 128, 128, causal=True)
+        mx, mean = attn_errors(out[:, h:h + 1], ref)
+        assert mx <= MAX_ABS and mean <= MEAN_ABS, (h, mx, mean)
+        assert float((lse[:, h:h + 1].cpu() - ref_lse).abs().max()) <= 5e-3
 
 
 def test_c5_gqa_ratio_7_forward_lse_backward_vs_oracle():
