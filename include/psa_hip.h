@@ -259,7 +259,7 @@ int64_t psa_fwd_workspace_bytes(int B, int Hq, int L, int block_m);
  * rows in index order - the same order in every run).  It is the counterpart of the reference's index list, which is
  * also computed once per map and then walked by the kernel:
  *   reference src/psa_triton/utils/transfer_attn_to_mask.py:271-500 (list built), src/psa_triton/kernels/psa_kernel.py:207-302 (walked).
- * Schedules exist for D = 128, block_m = block_n = 128 (psa_schedule_bytes returns 0 otherwise and psa_build_schedule
+ * Schedules exist for D = 64 or 128, block_m = block_n = 128 (psa_schedule_bytes returns 0 otherwise and psa_build_schedule
  * PSA_ERR_UNSUPPORTED; psa_fwd covers every shape).  `schedule`: caller-allocated device memory of psa_schedule_bytes(...)
  * bytes, 16-byte aligned (the bound is the worst case, every pair at level 1: 32 bytes per (q-block, kv-block) pair; only
  * the retained tiles are written and read).  It stays valid for as long as the map is unchanged and may be used by any

@@ -94,7 +94,9 @@ constexpr int F_ISTR = psa_tiles::LT_ISTR;  // bytes between the blocks of a til
     __syncthreads();                        \
   } while (0)
 
-template <int D, int NW, class ET>
+// GS: the row's tiles come from a prebuilt schedule (psa_schedule.h) as in the two-group kernel below: one scalar word
+// per wave and tile instead of a per-lane look-up, copies addressed from scalar registers.
+template <int D, int NW, bool GS, class ET>
 __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   using x8 = typename ET::x8;
   using G = psa_tiles::LtGeom<D>;
@@ -103,6 +105,7 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   constexpr int G16 = 4 / NW;  // 16-row groups of a tile fetched by one wave
   constexpr int OST = D * 2 + 16;
   static_assert(NW == 4 || NW == 2 || NW == 1, "1, 2 or 4 waves");
+  static_assert(!GS || NW == 4, "schedules describe 128-row q-blocks: one 16-row quarter of a tile per wave");
   static_assert(BM * OST <= 4 * F_TILE, "O staging must fit the tile buffers");
   const auto P_L = p.L;
   const auto P_bn_log2 = p.bn_log2;
@@ -147,8 +150,17 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const x8*)(qp + kk * 16);
   }
-  const int T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2,
-                                                 P_L, P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
+  using w_ptr = const __attribute__((address_space(4))) uint32_t*;
+  using rec_ptr = const __attribute__((address_space(4))) u32x4*;
+  rec_ptr recs = nullptr;
+  int T;
+  if constexpr (GS) {
+    recs = (rec_ptr)(uintptr_t)(p.sched_rec + (int64_t)logical * p.rec_stride);
+    T = __builtin_amdgcn_readfirstlane(p.sched_tiles[logical]);
+  } else {
+    T = psa_tiles::build_row_schedule<NT>(p.map, p.map_elem, ((int64_t)bh * p.Mq + I) * p.Nk, p.Nk, jmax, P_bn_log2, P_L,
+                                          P_causal != 0, (int64_t)I * p.bm, ids, tdesc, s_cnt, s_ioff, s_toff, s_wcnt);
+  }
 
   const char* kb0 = (const char*)(p.k + b * p.k_sb + hk * p.k_sh);
   const char* vb0 = (const char*)(p.v + b * p.v_sb + hk * p.v_sh);
@@ -179,10 +191,34 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   float l_run = 0.f;        // this lane's partial row sum
 
   // masks (if needed) and reduces the logits of tile t; returns the bias - reference max and the rescale factor
+  uint32_t w_cur = 0;  // GS: this wave's word of the record of the tile whose logits are being reduced
   auto softmax_head = [&](int t, f32x16 (&s_cur)[2], float& nb, float& alpha) __attribute__((always_inline)) {
-    const uint32_t d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
+    uint32_t d;
+    if constexpr (GS) d = ((w_cur >> psa_sched::REC_CODE_SHIFT) & 3u) | ((w_cur >> (psa_sched::REC_MASKED_BIT - 2)) & 4u);  // level | masked << 2
+    else d = __builtin_amdgcn_readfirstlane(tdesc[t][0]);
     const int lv = d & 3;
-    if (d & 4) {
+    if constexpr (GS) {
+      if (d & 4) {
+        const int nvalid = psa_sched::rec_nvalid(w_cur);
+        const int qlim = (q_idx + 1) >> lv;
+        u32x4 r4 = {0u, 0u, 0u, 0u};
+        if (P_causal) r4 = recs[t];  // the source rows of all four quarters (rare path: fetched on demand)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int r0 = c * 32 + g * 8 + hh * 4;
+            int keep = nvalid - r0;
+            if (P_causal) {
+              // slots r0 .. r0+3 lie in quarter 2c + g/2 of the tile, whose source rows are consecutive
+              const int src0 = psa_sched::rec_src(r4[c * 2 + (g >> 1)]) + (g & 1) * 8 + hh * 4;
+              keep = keep < qlim - src0 ? keep : qlim - src0;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s_cur[c][g * 4 + e] = e < keep ? s_cur[c][g * 4 + e] : -INFINITY;
+          }
+      }
+    } else if (d & 4) {
       // Partly empty tile and/or causal diagonal.  Valid slots are a prefix of the tile (nvalid), and a
       // pooled key of level lv is visible to query i once its last token is: ((src + 1) << lv) - 1 <= i, i.e.
       // src < (i + 1) >> lv.  Both limits cut each run of 4 consecutive slots after its first `keep` elements.
@@ -306,20 +342,74 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
   // Per tile: DMA tile t+1 | QK(t) | softmax(t) | PV(t) | barrier.  The MFMA phases of one workgroup overlap
   // the softmax of the other workgroup on the CU.  (Interleaving the exponentials of tile t with the MFMAs of
   // tiles t-1 / t+1 inside one wave was measured and is slower: it serialises the MFMA chains and costs registers.)
+  // GS: copies addressed from scalar registers (see the two-group kernel for the scheme)
+  const int lane_row = psa_tiles::lt_fetch_row<D>(lane);
+  const uint32_t voff_s = (uint32_t)lane_row * (uint32_t)(D * 2) + f_chunk;
+  const uint32_t wave_lds = psa_tiles::lds_addr_of(smem) + (uint32_t)(wave * G::RPL * F_ISTR);
+  auto pool_base = [&](const uint16_t* pool, int lv) __attribute__((always_inline)) {
+    return (const char*)pool + (BHkv * (P_npad - (P_npad >> (lv - 1))) + bhk * (P_npad >> lv)) * (D * 2);
+  };
+  struct Stream {  // where one tensor's tiles currently come from: a level's rows (the level changes 3 times per row)
+    const char* base;
+    uint32_t code;
+  };
+  Stream st_k = {kb0, 0u}, st_v = {vb0, 0u};
+  auto issue_tile = [&](Stream& st, bool is_k, uint32_t w, auto lds_byte) __attribute__((always_inline)) {
+    const uint32_t code = psa_sched::rec_code(w);
+    bool rag = false;
+    if (code != st.code) {
+      const int lv = (int)(code & 3u);
+      st.code = code & 3u;  // (a ragged tile comes back here for every tile)
+      const uint16_t* pool = is_k ? P_kp : P_vp;
+      st.base = lv == 0 ? (is_k ? kb0 : vb0) : pool_base(pool, lv);
+      rag = code == psa_sched::REC_CODE_RAGGED;
+    }
+    if (rag) {
+      static_for<G::RPL>([&](auto n) __attribute__((always_inline)) {
+        constexpr int N = decltype(n)::value, OFF = decltype(lds_byte)::value + N * F_ISTR;
+        const int row = psa_sched::rec_src(w) + lane_row + N;
+        psa_tiles::lds_copy16_row<OFF>(st.base, (uint32_t)(row < P_L - 1 ? row : P_L - 1), (uint32_t)(D * 2), f_chunk, wave_lds);
+      });
+    } else {
+      const char* src = st.base + (uint64_t)((w & psa_sched::REC_SRC_MASK) * (uint32_t)(D * 2));
+      static_for<G::RPL>([&](auto n) __attribute__((always_inline)) {
+        constexpr int N = decltype(n)::value;
+        psa_tiles::lds_copy16_imm<decltype(lds_byte)::value + N * F_ISTR, N * D * 2>(src, voff_s, wave_lds);
+      });
+    }
+  };
+
   if (T > 0) {
     TileSrc ts;
     f32x16 s[2];
     uint32_t pk[2][8];
-    tile_src(0, ts);
-    issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, 0);
-    issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, 2 * F_TILE);
+    w_ptr wp = nullptr;
+    uint32_t w_next = 0, w_next2 = 0;  // GS: words of tiles t+1 and t+2 (records T .. T+2 repeat record T-1)
+    if constexpr (GS) {
+      wp = (w_ptr)(uintptr_t)((const uint32_t*)(p.sched_rec + (int64_t)logical * p.rec_stride) + wave);
+      w_cur = wp[0];
+      w_next = wp[4];
+      w_next2 = wp[8];
+      wp += 12;
+      issue_tile(st_k, true, w_cur, IC<0>{});
+      issue_tile(st_v, false, w_cur, IC<2 * F_TILE>{});
+    } else {
+      tile_src(0, ts);
+      issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, 0);
+      issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, 2 * F_TILE);
+    }
     TILE_SYNC();
     auto step = [&](int t, auto cur_c) __attribute__((always_inline)) {
       constexpr int CUR = decltype(cur_c)::value;
       if (t + 1 < T) {
-        tile_src(t + 1, ts);
-        issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, (CUR ^ 1) * F_TILE);
-        issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, (2 + (CUR ^ 1)) * F_TILE);
+        if constexpr (GS) {
+          issue_tile(st_k, true, w_next, IC<(CUR ^ 1) * F_TILE>{});
+          issue_tile(st_v, false, w_next, IC<(2 + (CUR ^ 1)) * F_TILE>{});
+        } else {
+          tile_src(t + 1, ts);
+          issue_rows(ts.kbase, ts.kstr, ts.lim, ts.src0, (CUR ^ 1) * F_TILE);
+          issue_rows(ts.vbase, ts.vstr, ts.lim, ts.src0, (2 + (CUR ^ 1)) * F_TILE);
+        }
       }
       float nb, alpha, lsum = 0.f;
       qk_full(cur_c, s);
@@ -330,6 +420,12 @@ __global__ __launch_bounds__(NW * 64, 2) void psa_fwd_lds_kernel(FwdParams p) {
       rescale_acc(alpha);
       pv_half(cur_c, 0, pk[0]);
       pv_half(cur_c, 1, pk[1]);
+      if constexpr (GS) {
+        w_cur = w_next;
+        w_next = w_next2;
+        w_next2 = *wp;  // the word of tile t+3 (one scalar load; the records are padded, so no bounds test)
+        wp += 4;
+      }
       TILE_SYNC();
     };
     for (int t = 0; t < T; t += 2) {
@@ -954,18 +1050,19 @@ __global__ __launch_bounds__(2 * NW * 64, 1) void psa_fwd_pp_kernel(FwdParams p)
 }
 
 
-template <int D, int NW>
+template <int D, int NW, bool GS = false>
 int launch_fwd(const FwdParams& p, int Nk, hipStream_t stream) {
-  size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (size_t)p.max_tiles * 8 + (size_t)Nk * 2;
+  // with a prebuilt schedule the workgroup keeps nothing but its tile buffers in LDS
+  size_t shmem = (size_t)4 * psa_tiles::LtGeom<D>::TILE + (GS ? 0 : (size_t)p.max_tiles * 8 + (size_t)Nk * 2);
   if (shmem > 160 * 1024) return PSA_ERR_UNSUPPORTED;
   int rc = PSA_OK;
   psa_dispatch16(p.dtype, [&](auto et) {
     using ET = decltype(et);
-    if (hipFuncSetAttribute((const void*)psa_fwd_lds_kernel<D, NW, ET>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) {
+    if (hipFuncSetAttribute((const void*)psa_fwd_lds_kernel<D, NW, GS, ET>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess) {
       rc = PSA_ERR_LAUNCH;
       return;
     }
-    hipLaunchKernelGGL((psa_fwd_lds_kernel<D, NW, ET>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
+    hipLaunchKernelGGL((psa_fwd_lds_kernel<D, NW, GS, ET>), dim3((unsigned)(p.wg_chunk * p.wg_groups)), dim3(NW * 64), shmem, stream, p);
   });
   return rc;
 }
@@ -1075,11 +1172,11 @@ static int fwd_impl(psa_tensor4 q, psa_tensor4 k, psa_tensor4 v, const void* k_p
       p.sched_rec = (const u32x4*)(base + g.lay.rec_off);
       p.sched_tiles = (const int32_t*)(base + g.lay.tiles_off);
       p.rec_stride = g.lay.rec_stride;
-      rc = launch_fwd_pp<128, 4, true>(p, Nk, (hipStream_t)stream);
+      rc = D == 128 ? launch_fwd_pp<128, 4, true>(p, Nk, (hipStream_t)stream) : launch_fwd<64, 4, true>(p, Nk, (hipStream_t)stream);
     } else if (two_group) {
       rc = launch_fwd_pp<128, 4, false>(p, Nk, (hipStream_t)stream);
     } else {
-      rc = launch_fwd<128, 4>(p, Nk, (hipStream_t)stream);
+      rc = D == 128 ? launch_fwd<128, 4>(p, Nk, (hipStream_t)stream) : launch_fwd<64, 4>(p, Nk, (hipStream_t)stream);
     }
     PSA_REQUIRE(rc == PSA_OK, rc, "psa_fwd: sequence too long for the on-chip schedule (LDS)");
     return psa_check_launch("psa_fwd");

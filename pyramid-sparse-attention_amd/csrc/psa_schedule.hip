@@ -119,7 +119,7 @@ void psa_fwd_deal(int B, int Hq, int Hkv, int L, int D, int block_m, int block_n
 }
 
 bool psa_schedule_shape_ok(int D, int block_m, int block_n, int L) {
-  return D == 128 && block_m == 128 && block_n == 128 && (int64_t)((L + 127) / 128) * 128 <= (1 << psa_sched::REC_SRC_BITS);
+  return (D == 128 || D == 64) && block_m == 128 && block_n == 128 && (int64_t)((L + 127) / 128) * 128 <= (1 << psa_sched::REC_SRC_BITS);
 }
 
 bool psa_schedule_geometry(int B, int Hq, int Hkv, int L, int D, int block_m, int block_n, psa_sched::Geometry& g) {
@@ -145,7 +145,7 @@ extern "C" int psa_build_schedule(const void* map, int map_elem_bytes, void* sch
   PSA_REQUIRE(map_elem_bytes == 1 || map_elem_bytes == 4, PSA_ERR_ARG, "psa_build_schedule: map_elem_bytes must be 1 or 4");
   PSA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0 && Hq % Hkv == 0, PSA_ERR_ARG, "psa_build_schedule: bad B / H / L");
   PSA_REQUIRE(psa_schedule_shape_ok(D, block_m, block_n, L), PSA_ERR_UNSUPPORTED,
-              "psa_build_schedule: schedules exist for D = 128, block_m = block_n = 128 (got D=%d, block_m=%d, block_n=%d)", D, block_m, block_n);
+              "psa_build_schedule: schedules exist for D = 64 or 128, block_m = block_n = 128 (got D=%d, block_m=%d, block_n=%d)", D, block_m, block_n);
   PSA_REQUIRE((uintptr_t)schedule % 16 == 0, PSA_ERR_ARG, "psa_build_schedule: schedule must be 16-byte aligned");
   psa_sched::Geometry g;
   PSA_REQUIRE(psa_schedule_geometry(B, Hq, Hkv, L, D, block_m, block_n, g), PSA_ERR_UNSUPPORTED, "psa_build_schedule: shape out of range");

@@ -469,7 +469,7 @@ def density(level_map_: torch.Tensor, causal: bool = False) -> torch.Tensor:
 def build_schedule(level_map_: torch.Tensor, Hkv: int, L: int, D: int, block_m: int, block_n: int, causal: bool = False,
                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Tile schedule of a level map [B, Hq, Mq, Nk] (int8 / int32): a uint8 buffer for sparse_attention_fwd(schedule=...).
-    Exists for D = 128 and 128 x 128 blocks (ValueError otherwise)."""
+    Exists for D = 64 or 128 and 128 x 128 blocks (ValueError otherwise)."""
     _require_gpu(level_map_)
     if level_map_.dtype not in (torch.int8, torch.int32) or not level_map_.is_contiguous():
         raise ValueError("level map must be a contiguous int8/int32 tensor")

@@ -1,7 +1,8 @@
 """The prebuilt tile schedule (psa_build_schedule + psa_fwd_scheduled) against the walk that compacts the map row
 inside the kernel (psa_fwd): the schedule lists a row's tiles in the order the in-kernel builder produces them, so
 outputs and lse must be the same bits.  The in-kernel walk is the one the other forward tests compare with the oracle
-at shapes without a schedule; shapes with one reach the oracle through the schedule in test_gpu_fwd / test_gpu_configs."""
+at shapes without a schedule; shapes with one (head dim 64 or 128 with 128-token blocks) reach the oracle through the
+schedule in test_gpu_fwd / test_gpu_configs."""
 import numpy as np
 import pytest
 import torch
@@ -13,7 +14,7 @@ pytestmark = pytest.mark.gpu
 D, BM, BN = 128, 128, 128
 
 
-def _inputs(B, Hq, Hkv, L, seed):
+def _inputs(B, Hq, Hkv, L, seed, D=D):
     return (rnd(B, Hq, L, D, seed=seed).to(dev()), rnd(B, Hkv, L, D, seed=seed + 1).to(dev()), rnd(B, Hkv, L, D, seed=seed + 2).to(dev()))
 
 
@@ -31,10 +32,11 @@ def _inputs(B, Hq, Hkv, L, seed):
         (1, 1, 1, 4100, False, False, (0.9, 0.025, 0.025, 0.025, 0.025)),  # rows with very few tiles, empty rows
     ],
 )
-def test_scheduled_walk_equals_map_walk(B, Hq, Hkv, L, causal, indexed, p):
+@pytest.mark.parametrize("D", [128, 64])  # the two-group kernel / the one-row kernel
+def test_scheduled_walk_equals_map_walk(B, Hq, Hkv, L, causal, indexed, p, D):
     from psa_hip import ops
 
-    q, k, v = _inputs(B, Hq, Hkv, L, seed=L)
+    q, k, v = _inputs(B, Hq, Hkv, L, seed=L, D=D)
     Mq, Nk = -(-L // BM), -(-L // BN)
     lmap = torch.from_numpy(random_map(B, Hq, Mq, Nk, L + 7, p=p, ensure_row=False)).to(torch.int8).to(dev())
     qi = torch.randperm(L, generator=torch.Generator().manual_seed(L)).to(torch.int32).to(dev()) if indexed else None
@@ -72,7 +74,9 @@ def test_schedule_is_reusable_and_deterministic():
     ref, _ = O.psa_attention_dense(q.cpu(), k.cpu(), v.cpu(), lmap.cpu().numpy().astype(np.int32), BM, BN)
     mx, mean = attn_errors(outs[0], ref)
     assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
-    assert lib.psa_schedule_bytes(B, H, H, L, 64, BM, BN) == 0 and lib.psa_schedule_bytes(B, H, H, L, D, 64, BN) == 0
+    # schedules exist for head dims 64 and 128 with 128-token blocks
+    assert lib.psa_schedule_bytes(B, H, H, L, 64, BM, BN) > 0
+    assert lib.psa_schedule_bytes(B, H, H, L, 32, BM, BN) == 0 and lib.psa_schedule_bytes(B, H, H, L, D, 64, BN) == 0
 
 
 def test_strided_rows_fall_back_to_the_map_walk():
