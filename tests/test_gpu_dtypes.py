@@ -172,3 +172,27 @@ def test_layer_operator_fp16_pools_are_not_fed_to_the_bf16_backward():
     got = ops.sparse_attention_bwd(qd, kd, vd, lm, out, dod, lse, 128, 128, pools=pools16)
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_layer_operator_in_the_input_type_head_dim_128(dtype):
+    """The whole layer operator (estimate + map, pooling, tile schedule for the 16-bit types, forward) on fp16 / fp32
+    tensors with head dim 128 and 128-token blocks: scores, map and output against the oracle on the same values."""
+    from psa_hip import ops
+    from psa_hip.utils.synthetic import make_qkv, sample_offsets
+
+    B, H, D, bm, bn, tn = 1, 2, 128, 128, 128, 32
+    q, k, v = make_qkv(B, H, H, (3, 20, 26), D, seed=5, dtype=dtype)  # 1560 tokens, ragged last block
+    oq, ok = sample_offsets(B, H, bm, 32, 6), sample_offsets(B, H, bn, 32, 7)
+    ratios = {1: (0.0, 0.3), 2: (0.3, 0.45), 4: (0.45, 0.6), 8: (0.6, 0.8), 0: (0.8, 1.0)}
+    qd, kd, vd, oqd, okd = (t.to(dev()) for t in (q, k, v, oq, ok))
+    out, mp = ops.psa_layer_fwd(qd, kd, vd, oqd, okd, ratios, "thresholdbound", bm, bn, tn, return_map=True)
+    scores = ops.estimate_sampled(qd, kd, oqd, okd, bm, bn, 32, 32)
+    torch.cuda.synchronize()
+    assert out.dtype == dtype
+    np.testing.assert_allclose(scores.cpu().numpy(), O.estimate_sampled(q, k, bm, bn, oq, ok).numpy(), rtol=2e-4, atol=1e-9)
+    ref_map = O.level_map(scores.cpu().numpy(), ratios, 0, "thresholdbound", blocksize=bn, compute_tile=tn)
+    assert np.array_equal(mp.cpu().numpy(), ref_map)
+    ref, _ = O.psa_attention_blockwalk(q, k, v, ref_map, bm, bn)
+    mx, mean = attn_errors(out, ref)
+    assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], (mx, mean)
