@@ -89,40 +89,59 @@ def time_gpu(fn, iters, warm=20):
     return ts[len(ts) // 2], sum(ts) / len(ts)
 
 
-def sclk_under_load(fn, ms_per_call):
-    """Shader clock (MHz) that rocm-smi reports while fn runs back to back for about 1.5 s: the clock the launch's cycles
-    are counted in (the published peak is quoted at the 2400 MHz maximum).  None when rocm-smi gives no reading."""
+def load_telemetry(fn, ms_per_call, flops_per_call=0.0):
+    """What rocm-smi reports while fn runs back to back for about 3 s: the shader clock (the clock the launch's cycles are
+    counted in - the published peak is quoted at the 2400 MHz maximum), and the board's average power over the run from
+    its energy counter, with the energy per call (and per flop) that follows.  Fields are None where rocm-smi gives no
+    reading."""
     import re
     import subprocess
     import threading
 
     import torch
 
+    def smi(*args):
+        try:
+            return subprocess.run(["rocm-smi", *args], capture_output=True, text=True, timeout=20).stdout
+        except Exception:
+            return ""
+
+    def energy_uj():
+        m = re.search(r"Accumulated Energy \(uJ\):\s*([\d.]+)", smi("--showenergycounter"))
+        return float(m.group(1)) if m else None
+
     reads, stop = [], threading.Event()
 
     def poll():
         while not stop.is_set():
-            try:
-                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
-                m = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", out)
-                if m:
-                    reads.append(int(m.group(1)))
-            except Exception:
-                return
+            m = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", smi("--showclocks"))
+            if m:
+                reads.append(int(m.group(1)))
             stop.wait(0.1)
 
     th = threading.Thread(target=poll, daemon=True)
     for _ in range(20):
         fn()
     torch.cuda.synchronize()
+    n = max(10, int(3000.0 / max(ms_per_call, 1e-3)))
+    e0, t0 = energy_uj(), time.perf_counter()
     th.start()
-    for _ in range(max(10, int(1500.0 / max(ms_per_call, 1e-3)))):
+    for _ in range(n):
         fn()
     torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    e1 = energy_uj()
     stop.set()
     th.join(timeout=30)
     reads = sorted(reads[1:] or reads)  # (the first reading may predate the load)
-    return reads[len(reads) // 2] if reads else None
+    out = {"sclk_mhz": reads[len(reads) // 2] if reads else None, "avg_power_w": None, "joule_per_call": None, "pj_per_flop": None}
+    if e0 is not None and e1 is not None and e1 > e0:
+        joule = (e1 - e0) / 1e6
+        out["avg_power_w"] = round(joule / dt, 0)
+        out["joule_per_call"] = round(joule / n, 4)
+        if flops_per_call:
+            out["pj_per_flop"] = round(joule / n / flops_per_call * 1e12, 3)
+    return out
 
 
 def copy_calib(torch, dev):
@@ -400,18 +419,20 @@ def main():
         t_sched, _ = time_gpu(lambda: ops.build_schedule(mp, H, L, D, bm, bn, out=sched), it)
     fwd_call = lambda: ops.sparse_attention_fwd(q, k, v, mp, bm, bn, pools=(kp, vp), out=out_buf, schedule=sched)
     t_fwd_med, t_fwd_avg = time_gpu(fwd_call, it)
-    sclk = None if args.no_extras else sclk_under_load(fwd_call, t_fwd_avg)
+    exec_flops_fwd = 4.0 * L * L * D * H * B * float(ops.density(mp)[-1])
+    tele = None if args.no_extras else load_telemetry(fwd_call, t_fwd_avg, exec_flops_fwd)
+    sclk = tele["sclk_mhz"] if tele else None
     lib_gemm = None
     if not args.no_extras:
-        # context: what the vendor library's bf16 GEMM (torch.matmul, 8192^3) sustains on this box, and at which clock
+        # context: what the vendor library's bf16 GEMM (torch.matmul, 8192^3) sustains on this box, at which clock and power
         ga = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
         gb = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
         gemm_call = lambda: torch.matmul(ga, gb)
         _, t_gemm = time_gpu(gemm_call, 30)
         lib_gemm = {"what": "torch.matmul bf16 8192 x 8192 x 8192", "ms": round(t_gemm, 4),
                     "tflops": round(2.0 * 8192 ** 3 / (t_gemm * 1e-3) / 1e12, 1),
-                    "frac_of_peak": round(2.0 * 8192 ** 3 / (t_gemm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-                    "sclk_mhz_under_load": sclk_under_load(gemm_call, t_gemm)}
+                    "frac_of_peak": round(2.0 * 8192 ** 3 / (t_gemm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        lib_gemm.update(load_telemetry(gemm_call, t_gemm, 2.0 * 8192 ** 3))
         del ga, gb
     t_dense = t_sdpa = None
     if not args.no_dense:
@@ -485,6 +506,9 @@ def main():
         # the 2400 MHz the peak is quoted at) and the fraction of the peak scaled to that clock
         "sclk_mhz_under_load": sclk,
         "frac_at_that_clock": None if not sclk else round(exec_flops / (t_fwd_avg * 1e-3) / 1e12 / (peak * sclk / 2400.0), 4),
+        # board power while the kernel runs back to back (rocm-smi's energy counter; the board's cap is 1400 W)
+        "avg_power_w_under_load": tele["avg_power_w"] if tele else None,
+        "pj_per_flop": tele["pj_per_flop"] if tele else None,
         "launch_includes": ("the forward kernel alone (it walks the map's prebuilt tile schedule: stages_ms.schedule)" if sched is not None
                             else "the forward kernel and its two row-ordering launches"),
     }
